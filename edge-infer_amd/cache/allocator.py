@@ -111,12 +111,15 @@ class SequencePages:
 
     `window` None: a sequence keeps every page.  `window` w: after a step, pages
     that hold only positions no later query can see (position <= length - w)
-    are given back; their table entries read -1.
+    are given back; their table entries read -1.  `chunk` c: a query sees only keys of
+    its own block of c positions (counted from the sequence's start), so pages that lie
+    wholly before the block of the next position are given back as well.
     """
 
-    def __init__(self, pool: PagePool, n_slots: int, window=None):
+    def __init__(self, pool: PagePool, n_slots: int, window=None, chunk=None):
         self.pool = pool
         self.window = window
+        self.chunk = chunk
         self._pages: Dict[int, List[int]] = {}
         self._version: Dict[int, int] = {}     # counts the changes of a slot's page list
         self._changes = 0
@@ -148,9 +151,13 @@ class SequencePages:
 
     def trim(self, slot: int, length: int) -> None:
         """Give back pages wholly before the window of the next query."""
-        if self.window is None:
+        if self.window is None and self.chunk is None:
             return
-        first_visible = length - self.window + 1  # for the query at position `length`
+        first_visible = 0                         # for the query at position `length`
+        if self.window is not None:
+            first_visible = length - self.window + 1
+        if self.chunk is not None:
+            first_visible = max(first_visible, length // self.chunk * self.chunk)
         pages = self._pages[slot]
         dead = []
         for index, page in enumerate(pages):

@@ -76,7 +76,8 @@ class SessionCache:
         for request, entries in layout.kv_groups:
             pool = PagePool(self.n_pages)
             self.kv_pools.append(pool)
-            self.kv_pages.append(SequencePages(pool, self.n_slots, window=request.window))
+            self.kv_pages.append(SequencePages(pool, self.n_slots, window=request.window,
+                                               chunk=request.chunk))
             shape = (len(entries), self.n_pages, request.n_kv_heads, PAGE_TOKENS)
             value_dim = request.head_dim if request.value_dim is None else request.value_dim
             self.kv_k.append(torch.empty(shape + (request.head_dim,), dtype=dtype, device=device))

@@ -53,6 +53,9 @@ def resolve_architecture(config: Mapping[str, Any]) -> Architecture:
     names = config.get("architectures") or []
     if isinstance(names, str):
         names = [names]
+    single = config.get("architecture")      # some families name theirs under this key
+    if isinstance(single, str):
+        names = list(names) + [single]
     for name in names:
         if name in _ARCHITECTURES:
             return _ARCHITECTURES[name]

@@ -41,6 +41,22 @@ class AttentionSpec:
     window: Optional[int] = None   # None: every earlier key; w: the last w keys
     scale: Optional[float] = None  # None: 1/sqrt(head_dim)
     position: PositionSpec = field(default_factory=PositionSpec)
+    value_dim: Optional[int] = None     # None: values as wide as keys
+    # biases of the q, k and v projections: None: taken when the checkpoint holds them,
+    # True: the checkpoint must hold them, False: it must not
+    qkv_bias: Optional[bool] = None
+    # "head": RMSNorm of every head with one weight [head_dim]; "projection": one RMSNorm
+    # over all heads of q (and of k) together, weights [heads * head_dim]
+    qk_norm_scope: str = "head"
+    # positions i >= j see each other only if i // chunk == j // chunk, counted from the
+    # sequence's position 0 (None: no such blocks)
+    chunk: Optional[int] = None
+    # r: the score of query i and key j is lowered by 2^(-r (h + 1) / heads) * (i - j) for
+    # head h (None: no distance term)
+    distance_slope_range: Optional[float] = None
+    # a learned number per head that joins the softmax's denominator as exp(sink), with no
+    # key and no value
+    sink: bool = False
 
     @property
     def q_width(self) -> int:
@@ -49,6 +65,25 @@ class AttentionSpec:
     @property
     def kv_width(self) -> int:
         return self.n_kv_heads * self.head_dim
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
+
+    @property
+    def v_width(self) -> int:
+        return self.n_kv_heads * self.v_dim
+
+    @property
+    def out_width(self) -> int:
+        return self.n_heads * self.v_dim
+
+    @property
+    def extended(self) -> bool:
+        """Whether the mixer uses anything beyond rotary/windowed attention with per-head
+        norms and equal widths (what the matrix-core kernels take)."""
+        return (self.v_dim != self.head_dim or self.qk_norm_scope != "head"
+                or self.chunk is not None or self.distance_slope_range is not None or self.sink)
 
 
 @dataclass(frozen=True)
@@ -60,11 +95,42 @@ class GatedMLPSpec:
 
 
 @dataclass(frozen=True)
+class DenseMLPSpec:
+    """down(act(up(x))); activation "relu2" (the square of relu), "relu", "silu" or
+    "gelu_tanh"."""
+    kind: str = "dense_mlp"
+    intermediate_size: int = 0
+    activation: str = "relu2"
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """Gated delta rule: a recurrent mixer whose state is one [key_dim, value_dim] matrix per
+    head, fed through short causal convolutions.  See `parts.delta`."""
+    kind: str = "gated_delta"
+    n_heads: int = 0              # value heads (one state each)
+    n_kv_heads: int = 0           # query/key heads, shared by n_heads / n_kv_heads value heads
+    key_dim: int = 0
+    value_dim: int = 0
+    conv_taps: int = 4            # taps of the causal convolution of q, k and v
+    out_norm_eps: float = 1e-6    # eps of the RMS norm of each head's read-out
+    unit_eps: float = 1e-6        # q and k become x / sqrt(sum(x^2) + unit_eps) per head
+
+    @property
+    def qk_width(self) -> int:
+        return self.n_kv_heads * self.key_dim
+
+    @property
+    def v_width(self) -> int:
+        return self.n_heads * self.value_dim
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     block: str            # arrangement, e.g. "prenorm"
     norm: NormSpec
     mixer: object         # a spec with a .kind (AttentionSpec, or one a test registers)
-    feed_forward: object  # a spec with a .kind (GatedMLPSpec, ...)
+    feed_forward: object  # a spec with a .kind (GatedMLPSpec, ...), or None: no feed-forward
 
 
 @dataclass(frozen=True)
@@ -86,8 +152,8 @@ class ModelSpec:
     final_norm: NormSpec
     tie_word_embeddings: bool
     max_position_embeddings: int
-    bos_token_id: int
-    eos_token_id: int
+    bos_token_id: Optional[int]   # None: the architecture names no such token
+    eos_token_id: Optional[int]
 
     def validate(self) -> None:
         if not self.layers or not self.schedule:

@@ -1,5 +1,5 @@
-// Causal grouped-query attention over the paged cache, any head size that is a
-// multiple of 16 up to 256, any head and group counts, float32 or bfloat16
+// Causal grouped-query attention over the paged cache, any key and value head size up to
+// 256 (the two may differ), any head and group counts, float32 or bfloat16
 // storage, float32 arithmetic throughout (scores, running maximum, exponentials,
 // sums and the value accumulation).  One kernel serves prefill (many positions of a
 // sequence) and decode (one position, the key range split over several blocks and
@@ -8,6 +8,9 @@
 // Mathematics of the reference: s_t = (q . k_t) / sqrt(d) for keys t <= p (and
 // t > p - window when a window is set), streaming softmax with a running maximum,
 // o = sum w_t v_t / sum w_t; query head h reads kv head h / (nq / nkv).
+// Options beyond the reference: `chunk` (a query at p sees key t only if t / chunk == p / chunk),
+// `slopes` (per query head: the score is lowered by slope * (p - t)), `sinks` (per query head:
+// exp(sink) joins the denominator; it has no key and no value).
 // operators/src/cuda/execution.cu:137-179, runtime/src/qwen.cpp:374-402,
 // split merge: operators/src/cuda/kernels/gather_fa_variable.cu:14-118.
 #include "common.h"
@@ -26,13 +29,15 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                     const int32_t* __restrict__ item_row0, const int32_t* __restrict__ item_npos,
                     const int32_t* __restrict__ row_pos, const int32_t* __restrict__ page_table,
                     int table_width, T* __restrict__ out, float* __restrict__ part_o,
-                    float* __restrict__ part_ml, int nq, int nkv, int D, int Gb, int head_blocks,
-                    int BC, int window, float scale, int n_splits) {
+                    float* __restrict__ part_ml, int nq, int nkv, int D, int DV, int Gb,
+                    int head_blocks, int BC, int window, int chunk,
+                    const float* __restrict__ slopes, const float* __restrict__ sinks,
+                    float scale, int n_splits) {
   extern __shared__ float lds[];
   float* Qs = lds;                        // [kRows][D]
   float* Ks = Qs + kRows * D;             // [BC][D + 1]
-  float* Vs = Ks + BC * (D + 1);          // [BC][D]
-  float* Ps = Vs + BC * D;                // [kRows][BC + 1]
+  float* Vs = Ks + BC * (D + 1);          // [BC][DV]
+  float* Ps = Vs + BC * DV;               // [kRows][BC + 1]
 
   const int item = blockIdx.x;
   const int g = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
@@ -49,6 +54,8 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
   const int head = g * G + head_in_group;
   const int row = row0 + pi;
   const int pos_r = row_valid ? row_pos[row] : -1;
+  const float slope = (slopes && row_valid) ? slopes[head] : 0.f;
+  const int chunk_r = (chunk > 0 && row_valid) ? pos_r / chunk : 0;
 
   // query rows, pre-scaled
   for (int idx = t; idx < kRows * D; idx += kThreads) {
@@ -64,12 +71,13 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
   float acc[16];
 #pragma unroll
   for (int k = 0; k < 16; ++k) acc[k] = 0.f;
-  const int nd = D / 16;
+  const int nd = (DV + 15) / 16;
   const int nj = BC / 16;
 
   if (seq >= 0 && npos > 0) {
     const int hi_key = row_pos[row0 + npos - 1];
-    const int lo_key = window > 0 ? max(0, row_pos[row0] - window + 1) : 0;
+    int lo_key = window > 0 ? max(0, row_pos[row0] - window + 1) : 0;
+    if (chunk > 0) lo_key = max(lo_key, row_pos[row0] / chunk * chunk);
     const int lo_page = lo_key / EI_PAGE, hi_page = hi_key / EI_PAGE;
     const int total_pages = hi_page - lo_page + 1;
     const int per = (total_pages + n_splits - 1) / n_splits;
@@ -80,17 +88,23 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
       const int phys = page_table[static_cast<size_t>(seq) * table_width + p];
       if (phys < 0) continue;  // a page the window has released: every key in it is masked
       const T* kp = k_pages + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
-      const T* vp = v_pages + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
+      const T* vp = v_pages + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * DV;
       for (int ch = 0; ch < chunks_per_page; ++ch) {
         const int key0 = p * EI_PAGE + ch * BC;
         if (key0 > hi_key) break;
+        if (key0 + BC <= lo_key) continue;   // wholly before what any row of the item sees
         __syncthreads();
         for (int idx = t; idx < BC * D; idx += kThreads) {
           const int c = idx / D, d = idx % D;
           const bool live = key0 + c <= hi_key;  // later slots hold stale bytes
           const size_t off = static_cast<size_t>(ch * BC + c) * D + d;
           Ks[c * (D + 1) + d] = live ? ei::to_f32<T>(kp[off]) : 0.f;
-          Vs[c * D + d] = live ? ei::to_f32<T>(vp[off]) : 0.f;
+        }
+        for (int idx = t; idx < BC * DV; idx += kThreads) {
+          const int c = idx / DV, d = idx % DV;
+          const bool live = key0 + c <= hi_key;
+          const size_t off = static_cast<size_t>(ch * BC + c) * DV + d;
+          Vs[c * DV + d] = live ? ei::to_f32<T>(vp[off]) : 0.f;
         }
         __syncthreads();
         float s[4];
@@ -101,12 +115,14 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
           if (j < nj) {
             const int c = cc + 16 * j;
             const int key = key0 + c;
-            const bool visible = row_valid && key <= pos_r && (window <= 0 || key > pos_r - window);
+            const bool visible = row_valid && key <= pos_r && (window <= 0 || key > pos_r - window) &&
+                                 (chunk <= 0 || key / chunk == chunk_r);
             if (visible) {
               float dot = 0.f;
               const float* qr = Qs + r * D;
               const float* kr = Ks + c * (D + 1);
               for (int d = 0; d < D; ++d) dot += qr[d] * kr[d];
+              dot -= slope * static_cast<float>(pos_r - key);
               s[j] = dot;
               row_max = fmaxf(row_max, dot);
             }
@@ -137,7 +153,8 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
           if (k < nd) {
             const int d = cc + 16 * k;
             float a = acc[k] * alpha;
-            for (int c = 0; c < BC; ++c) a += pr[c] * Vs[c * D + d];
+            if (d < DV)
+              for (int c = 0; c < BC; ++c) a += pr[c] * Vs[c * DV + d];
             acc[k] = a;
           }
         }
@@ -146,18 +163,28 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
   }
 
   if (!row_valid) return;
+  if (sinks && split == 0) {
+    // the sink is one more term of the denominator: exp(sink), on the row's running scale
+    const float sink = sinks[head];
+    const float m_new = fmaxf(m_r, sink);
+    const float alpha = expf(m_r - m_new);
+    l_r = l_r * alpha + expf(sink - m_new);
+#pragma unroll
+    for (int k = 0; k < 16; ++k) acc[k] *= alpha;
+    m_r = m_new;
+  }
   if (n_splits == 1) {
     const float inv = l_r > 0.f ? 1.f / l_r : 0.f;
-    T* dst = out + (static_cast<size_t>(row) * nq + head) * D;
+    T* dst = out + (static_cast<size_t>(row) * nq + head) * DV;
 #pragma unroll
     for (int k = 0; k < 16; ++k)
-      if (k < nd) dst[cc + 16 * k] = ei::from_f32<T>(acc[k] * inv);
+      if (k < nd && cc + 16 * k < DV) dst[cc + 16 * k] = ei::from_f32<T>(acc[k] * inv);
   } else {
     const size_t slot = (static_cast<size_t>(row) * nq + head) * n_splits + split;
-    float* dst = part_o + slot * D;
+    float* dst = part_o + slot * DV;
 #pragma unroll
     for (int k = 0; k < 16; ++k)
-      if (k < nd) dst[cc + 16 * k] = acc[k];
+      if (k < nd && cc + 16 * k < DV) dst[cc + 16 * k] = acc[k];
     if (cc == 0) {
       part_ml[slot * 2] = m_r;
       part_ml[slot * 2 + 1] = l_r;
@@ -202,19 +229,22 @@ extern "C" int ei_attn_positions_per_item(int G) {
   return kRows / gb;
 }
 
-// q, out: [N, nq, D]; pages: [n_pages, nkv, 64, D]; items: see the kernel.
-// n_splits > 1 needs part_o [N, nq, n_splits, D] and part_ml [N, nq, n_splits, 2]
+// q: [N, nq, D], out: [N, nq, DV]; key pages: [n_pages, nkv, 64, D], value pages:
+// [n_pages, nkv, 64, DV]; items: see the kernel.  chunk 0, slopes and sinks null: none.
+// n_splits > 1 needs part_o [N, nq, n_splits, DV] and part_ml [N, nq, n_splits, 2]
 // float32 and items that hold one position each (decode); the merge follows.
 extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pages, int dtype,
                             const int32_t* item_seq, const int32_t* item_row0,
                             const int32_t* item_npos, int n_items, const int32_t* row_pos,
                             const int32_t* row_seq, const int32_t* page_table, int table_width,
                             void* out, float* part_o, float* part_ml, int N, int nq, int nkv,
-                            int D, int window, float scale, int n_splits, hipStream_t stream) {
+                            int D, int DV, int window, int chunk, const float* slopes,
+                            const float* sinks, float scale, int n_splits, hipStream_t stream) {
   EI_REQUIRE(n_items > 0 && N > 0 && nq > 0 && nkv > 0, "attention: sizes must be positive");
   EI_REQUIRE(nq % nkv == 0, "attention: query heads must be a multiple of kv heads");
-  EI_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256,
-             "attention: head_dim must be a multiple of 16 between 16 and 256");
+  EI_REQUIRE(D >= 1 && D <= 256 && DV >= 1 && DV <= 256,
+             "attention: key and value head sizes must lie between 1 and 256");
+  EI_REQUIRE(chunk >= 0, "attention: negative chunk");
   EI_REQUIRE(q && k_pages && v_pages && out && item_seq && item_row0 && item_npos && row_pos &&
                  page_table && table_width > 0,
              "attention: null pointer");
@@ -224,24 +254,24 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
   const int G = nq / nkv;
   const int Gb = G < kRows ? G : kRows;
   const int head_blocks = (G + Gb - 1) / Gb;
-  const int BC = chunk_keys(D);
+  const int BC = chunk_keys(D > DV ? D : DV);
   const size_t lds =
       sizeof(float) * (static_cast<size_t>(kRows) * D + static_cast<size_t>(BC) * (D + 1) +
-                       static_cast<size_t>(BC) * D + static_cast<size_t>(kRows) * (BC + 1));
+                       static_cast<size_t>(BC) * DV + static_cast<size_t>(kRows) * (BC + 1));
   EI_REQUIRE(static_cast<long long>(nkv) * head_blocks <= 65535, "attention: too many heads");
   dim3 grid(n_items, nkv * head_blocks, n_splits);
   if (dtype == EI_F32) {
     attn_generic_kernel<float><<<grid, kThreads, lds, stream>>>(
         static_cast<const float*>(q), static_cast<const float*>(k_pages),
         static_cast<const float*>(v_pages), item_seq, item_row0, item_npos, row_pos, page_table,
-        table_width, static_cast<float*>(out), part_o, part_ml, nq, nkv, D, Gb, head_blocks, BC,
-        window, scale, n_splits);
+        table_width, static_cast<float*>(out), part_o, part_ml, nq, nkv, D, DV, Gb, head_blocks,
+        BC, window, chunk, slopes, sinks, scale, n_splits);
   } else if (dtype == EI_BF16) {
     attn_generic_kernel<bf16_t><<<grid, kThreads, lds, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
         static_cast<const bf16_t*>(v_pages), item_seq, item_row0, item_npos, row_pos, page_table,
-        table_width, static_cast<bf16_t*>(out), part_o, part_ml, nq, nkv, D, Gb, head_blocks, BC,
-        window, scale, n_splits);
+        table_width, static_cast<bf16_t*>(out), part_o, part_ml, nq, nkv, D, DV, Gb, head_blocks,
+        BC, window, chunk, slopes, sinks, scale, n_splits);
   } else {
     EI_REQUIRE(false, "attention: unknown dtype");
   }
@@ -256,10 +286,10 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
     const int blocks = (total * EI_WAVE + threads - 1) / threads;
     if (dtype == EI_F32)
       attn_merge_kernel<float><<<blocks, threads, 0, stream>>>(
-          part_o, part_ml, row_seq, static_cast<float*>(out), nq, D, n_splits, total);
+          part_o, part_ml, row_seq, static_cast<float*>(out), nq, DV, n_splits, total);
     else
       attn_merge_kernel<bf16_t><<<blocks, threads, 0, stream>>>(
-          part_o, part_ml, row_seq, static_cast<bf16_t*>(out), nq, D, n_splits, total);
+          part_o, part_ml, row_seq, static_cast<bf16_t*>(out), nq, DV, n_splits, total);
   }
   EI_LAUNCH_CHECK();
 }

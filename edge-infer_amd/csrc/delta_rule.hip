@@ -1,0 +1,407 @@
+// Gated delta rule: a recurrent mixer whose state is one matrix S [D, DV] per head and
+// sequence, fed through short causal convolutions.  Per token t and head h (query/key head
+// h / (H / G)), everything in float32:
+//
+//   x      = silu(conv(projection))          for the q, k and v channels (J taps a channel,
+//                                            the last one on the current token, zeros before
+//                                            the sequence starts)
+//   q, k   = x / sqrt(sum(x^2) + unit_eps)   per head; q also times q_scale
+//   beta   = sigmoid(b),  g = exp(-exp(A_log) * softplus(a + dt_bias))
+//   S     <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//   out    = o / sqrt(mean(o^2) + eps) * w * silu(gate)
+//
+// Per sequence the cache keeps S (stored transposed, [H, DV, D], so that the D values a
+// thread owns are contiguous) and the last J - 1 inputs of every convolved channel.  One
+// set of kernels serves prompts (rows of a sequence are walked in order) and decoding (one
+// row a sequence):
+//
+//   delta_conv   convolution + silu of all q, k, v channels of every row
+//   delta_tail   the new last J - 1 inputs of every sequence (after delta_conv has read the
+//                old ones)
+//   delta_rule   the recurrence; a thread owns 8 rows of one column of S, L = D / 8 lanes
+//                share a column; tokens come in tiles through LDS
+//   delta_out    the read-out's norm and gate
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kTile = 32;        // most tokens of a sequence that delta_rule stages in LDS at a time
+constexpr int kOwn = 8;          // rows of a column of S that one thread owns
+constexpr int kMaxTaps = 32;
+
+template <typename TI>
+__device__ __forceinline__ float slice_sum(const TI* p, int nsplit, size_t stride) {
+  float x = 0.f;
+  for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TI>(p[s * stride]);
+  return x;
+}
+
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+
+__device__ __forceinline__ float softplus_f32(float x) {
+  return x > 30.f ? x : log1pf(expf(x));
+}
+
+// proj: [nsplit][N, WP]; the convolved channels are its first C columns.  conv_w: [C, J].
+// The tail of a sequence (its last J - 1 inputs before this step, oldest first) lies at
+// state + slot * state_stride + tail_offset as [J - 1, C].
+template <typename TI>
+__global__ void delta_conv_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
+                                  int WP, const float* __restrict__ conv_w, int J,
+                                  const float* __restrict__ state, size_t state_stride,
+                                  size_t tail_offset, const int32_t* __restrict__ row_pos,
+                                  const int32_t* __restrict__ row_seq,
+                                  const int32_t* __restrict__ seq_slot,
+                                  const int32_t* __restrict__ seq_start, float* __restrict__ out,
+                                  size_t total, int C) {
+  const size_t first = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t idx = first; idx < total; idx += step) {
+    const size_t row = idx / C;
+    const int c = static_cast<int>(idx % C);
+    const int seq = row_seq[row];
+    if (seq < 0) continue;
+    const int pos = row_pos[row], start = seq_start[seq];
+    const float* tail = state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+    float acc = 0.f;
+    for (int j = 0; j < J; ++j) {
+      const int back = J - 1 - j;
+      const int p = pos - back;
+      float x = 0.f;
+      if (p >= start)
+        x = slice_sum(proj + (row - back) * WP + c, nsplit, split_stride);
+      else if (p >= 0)
+        x = tail[static_cast<size_t>(p - start + J - 1) * C + c];
+      acc += conv_w[static_cast<size_t>(c) * J + j] * x;
+    }
+    out[idx] = silu_f32(acc);
+  }
+}
+
+// The thread of a sequence's last row of the step writes the sequence's new tail for its
+// channel: the inputs of the last J - 1 positions, from this step's rows or, where the step
+// brought fewer, from the old tail (read before anything is written).
+template <typename TI>
+__global__ void delta_tail_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
+                                  int WP, int J, float* __restrict__ state, size_t state_stride,
+                                  size_t tail_offset, const int32_t* __restrict__ row_pos,
+                                  const int32_t* __restrict__ row_seq,
+                                  const int32_t* __restrict__ seq_slot,
+                                  const int32_t* __restrict__ seq_start,
+                                  const int32_t* __restrict__ seq_count, size_t total, int C) {
+  const size_t first = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t idx = first; idx < total; idx += step) {
+    const size_t row = idx / C;
+    const int c = static_cast<int>(idx % C);
+    const int seq = row_seq[row];
+    if (seq < 0) continue;
+    const int start = seq_start[seq], count = seq_count[seq];
+    if (row_pos[row] != start + count - 1) continue;
+    float* tail = state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+    float keep[kMaxTaps - 1];
+    for (int i = 0; i < J - 1; ++i) {
+      const int back = J - 2 - i;               // the input `back` positions before the last row
+      keep[i] = back < count ? slice_sum(proj + (row - back) * WP + c, nsplit, split_stride)
+                             : tail[static_cast<size_t>(i + count) * C + c];
+    }
+    for (int i = 0; i < J - 1; ++i) tail[static_cast<size_t>(i) * C + c] = keep[i];
+  }
+}
+
+// Sum over the L neighbouring lanes that share a column (L a power of two up to 32), every
+// one of them getting it.  Steps inside a row of 16 lanes are DPP modifiers of the add.
+template <int L>
+__device__ __forceinline__ float group_sum(float v) {
+  if (L >= 2)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xb1, 0xf, 0xf, false));
+  if (L >= 4)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4e, 0xf, 0xf, false));
+  if (L >= 8)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));
+  if (L >= 16)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));
+  if (L >= 32) {
+    const ei::ei_u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r.x) + __uint_as_float(r.y);
+  }
+  return v;
+}
+
+// conv: [N, C] = q [G * D] | k [G * D] | v [H * DV] after convolution and silu.  The block
+// (sequence, head, column block) walks the sequence's rows of this step in order.
+template <typename TI, int L>
+__global__ void __launch_bounds__(kThreads)
+delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ proj, int nsplit,
+                  size_t split_stride, int WP, int beta_col, int decay_col,
+                  const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                  float* __restrict__ state, size_t state_stride,
+                  const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ seq_count,
+                  const int32_t* __restrict__ seq_row0, float* __restrict__ o_raw, int H, int G,
+                  int D, int DV, float q_scale, float unit_eps) {
+  constexpr int DP = L * kOwn;            // D rounded up to what the lanes of a column hold
+  constexpr int CB = kThreads / L;        // columns of S a block holds
+  constexpr int TILE = L >= 32 ? kTile / 2 : kTile;   // (the widest keys: half, to fit 64 KB)
+  __shared__ __attribute__((aligned(16))) float q_s[TILE][DP];
+  __shared__ __attribute__((aligned(16))) float k_s[TILE][DP];
+  __shared__ float v_s[TILE][CB];
+  __shared__ float beta_s[kTile], decay_s[kTile], qf_s[kTile], kf_s[kTile];
+
+  const int seq = blockIdx.x;
+  const int count = seq_count[seq];
+  if (count <= 0) return;                 // padding of a fixed-size batch
+  const int row0 = seq_row0[seq];
+  const int head = blockIdx.y, shared_head = head / (H / G);
+  const int tid = threadIdx.x;
+  const int col_in_block = tid / L, part = tid % L;
+  const int col = blockIdx.z * CB + col_in_block;
+  const bool col_ok = col < DV;
+  const int i0 = part * kOwn;
+  const int QK = G * D, VW = H * DV;
+
+  float* mine = state + static_cast<size_t>(seq_slot[seq]) * state_stride +
+                (static_cast<size_t>(head) * DV + (col_ok ? col : 0)) * D + i0;
+  float s[kOwn];
+#pragma unroll
+  for (int m = 0; m < kOwn; ++m) s[m] = (col_ok && i0 + m < D) ? mine[m] : 0.f;
+  const float rate = expf(a_log[head]), shift = dt_bias[head];
+
+  for (int t0 = 0; t0 < count; t0 += TILE) {
+    const int nt = min(TILE, count - t0);
+    __syncthreads();                      // the last tile has been read
+    for (int idx = tid; idx < nt * DP; idx += kThreads) {
+      const int tt = idx / DP, i = idx % DP;
+      const float* src = conv + static_cast<size_t>(row0 + t0 + tt) * C + shared_head * D + i;
+      q_s[tt][i] = i < D ? src[0] : 0.f;
+      k_s[tt][i] = i < D ? src[QK] : 0.f;
+    }
+    for (int idx = tid; idx < nt * CB; idx += kThreads) {
+      const int tt = idx / CB, jj = idx % CB;
+      const int cg = blockIdx.z * CB + jj;
+      v_s[tt][jj] = cg < DV ? conv[static_cast<size_t>(row0 + t0 + tt) * C + 2 * QK + head * DV + cg]
+                            : 0.f;
+    }
+    if (tid < nt) {
+      const TI* src = proj + static_cast<size_t>(row0 + t0 + tid) * WP;
+      const float b = slice_sum(src + beta_col + head, nsplit, split_stride);
+      const float a = slice_sum(src + decay_col + head, nsplit, split_stride);
+      beta_s[tid] = 1.0f / (1.0f + expf(-b));
+      decay_s[tid] = expf(-rate * softplus_f32(a + shift));
+    }
+    __syncthreads();
+    {   // the factors that make q and k unit vectors: 8 threads a token
+      const int tt = tid / 8, sub = tid % 8;
+      float q_sq = 0.f, k_sq = 0.f;
+      if (tt < nt)
+        for (int i = sub; i < D; i += 8) {
+          q_sq += q_s[tt][i] * q_s[tt][i];
+          k_sq += k_s[tt][i] * k_s[tt][i];
+        }
+      q_sq = group_sum<8>(q_sq);
+      k_sq = group_sum<8>(k_sq);
+      if (tt < nt && sub == 0) {
+        qf_s[tt] = q_scale / sqrtf(q_sq + unit_eps);
+        kf_s[tt] = 1.0f / sqrtf(k_sq + unit_eps);
+      }
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float g = decay_s[tt], kf = kf_s[tt];
+      float kv[kOwn], qv[kOwn];
+      *reinterpret_cast<float4*>(kv) = *reinterpret_cast<const float4*>(&k_s[tt][i0]);
+      *reinterpret_cast<float4*>(kv + 4) = *reinterpret_cast<const float4*>(&k_s[tt][i0 + 4]);
+      *reinterpret_cast<float4*>(qv) = *reinterpret_cast<const float4*>(&q_s[tt][i0]);
+      *reinterpret_cast<float4*>(qv + 4) = *reinterpret_cast<const float4*>(&q_s[tt][i0 + 4]);
+      float seen0 = 0.f, seen1 = 0.f;
+#pragma unroll
+      for (int m = 0; m < kOwn; m += 2) {
+        s[m] *= g;
+        s[m + 1] *= g;
+        seen0 += s[m] * kv[m];
+        seen1 += s[m + 1] * kv[m + 1];
+      }
+      const float seen = group_sum<L>(seen0 + seen1) * kf;       // (S^T k)[col], k a unit vector
+      const float u = beta_s[tt] * (v_s[tt][col_in_block] - seen) * kf;
+      float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int m = 0; m < kOwn; m += 2) {
+        s[m] += kv[m] * u;
+        s[m + 1] += kv[m + 1] * u;
+        o0 += s[m] * qv[m];
+        o1 += s[m + 1] * qv[m + 1];
+      }
+      const float o = group_sum<L>(o0 + o1) * qf_s[tt];
+      if (part == 0 && col_ok)
+        o_raw[static_cast<size_t>(row0 + t0 + tt) * VW + head * DV + col] = o;
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int m = 0; m < kOwn; ++m)
+      if (i0 + m < D) mine[m] = s[m];
+  }
+}
+
+// One wave per (row, head): out = o / sqrt(mean(o^2) + eps) * w * silu(gate).
+template <typename TI, typename TO>
+__global__ void delta_out_kernel(const float* __restrict__ o_raw, const TI* __restrict__ proj,
+                                 int nsplit, size_t split_stride, int WP, int gate_col,
+                                 const float* __restrict__ norm_w, float eps,
+                                 const int32_t* __restrict__ row_seq, TO* __restrict__ out,
+                                 long long items, int H, int DV) {
+  const long long item = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) / EI_WAVE;
+  const int lane = threadIdx.x % EI_WAVE;
+  if (item >= items) return;
+  const long long row = item / H;
+  const int head = static_cast<int>(item % H);
+  const size_t base = static_cast<size_t>(row) * H * DV + static_cast<size_t>(head) * DV;
+  if (row_seq[row] < 0) {                 // padding row: a defined input for the next product
+    for (int j = lane; j < DV; j += EI_WAVE) out[base + j] = ei::from_f32<TO>(0.f);
+    return;
+  }
+  float sq = 0.f;
+  for (int j = lane; j < DV; j += EI_WAVE) sq += o_raw[base + j] * o_raw[base + j];
+  sq = ei::wave_sum(sq);
+  const float inv = 1.0f / sqrtf(sq / static_cast<float>(DV) + eps);
+  const TI* gate = proj + static_cast<size_t>(row) * WP + gate_col + static_cast<size_t>(head) * DV;
+  for (int j = lane; j < DV; j += EI_WAVE) {
+    const float gt = slice_sum(gate + j, nsplit, split_stride);
+    out[base + j] = ei::from_f32<TO>((o_raw[base + j] * inv) * norm_w[j] * silu_f32(gt));
+  }
+}
+
+int lanes_a_column(int D) {
+  int lanes = 1;
+  while (lanes * kOwn < D) lanes *= 2;
+  return lanes;
+}
+
+unsigned grid_for(size_t total) {
+  size_t blocks = (total + kThreads - 1) / kThreads;
+  const size_t most = static_cast<size_t>(ei_compute_units()) * 32;
+  return static_cast<unsigned>(blocks > most ? most : blocks);
+}
+
+}  // namespace
+
+extern "C" int ei_delta_conv(const void* proj, int in_dtype, int nsplit, long long split_stride,
+                             int WP, const float* conv_w, int J, const float* state,
+                             long long state_stride, long long tail_offset, const int32_t* row_pos,
+                             const int32_t* row_seq, const int32_t* seq_slot,
+                             const int32_t* seq_start, float* out, int N, int C,
+                             hipStream_t stream) {
+  EI_REQUIRE(proj && conv_w && state && row_pos && row_seq && seq_slot && seq_start && out,
+             "delta_conv: null pointer");
+  EI_REQUIRE(N > 0 && C > 0 && C <= WP && nsplit >= 1, "delta_conv: sizes must be positive");
+  EI_REQUIRE(J >= 1 && J <= kMaxTaps, "delta_conv: taps must lie between 1 and 32");
+  const size_t total = static_cast<size_t>(N) * C;
+  const size_t ss = static_cast<size_t>(split_stride);
+  if (in_dtype == EI_F32)
+    delta_conv_kernel<float><<<grid_for(total), kThreads, 0, stream>>>(
+        static_cast<const float*>(proj), nsplit, ss, WP, conv_w, J, state,
+        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
+        seq_slot, seq_start, out, total, C);
+  else if (in_dtype == EI_BF16)
+    delta_conv_kernel<bf16_t><<<grid_for(total), kThreads, 0, stream>>>(
+        static_cast<const bf16_t*>(proj), nsplit, ss, WP, conv_w, J, state,
+        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
+        seq_slot, seq_start, out, total, C);
+  else
+    EI_REQUIRE(false, "delta_conv: unknown dtype");
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_delta_tail(const void* proj, int in_dtype, int nsplit, long long split_stride,
+                             int WP, int J, float* state, long long state_stride,
+                             long long tail_offset, const int32_t* row_pos, const int32_t* row_seq,
+                             const int32_t* seq_slot, const int32_t* seq_start,
+                             const int32_t* seq_count, int N, int C, hipStream_t stream) {
+  EI_REQUIRE(proj && state && row_pos && row_seq && seq_slot && seq_start && seq_count,
+             "delta_tail: null pointer");
+  EI_REQUIRE(N > 0 && C > 0 && C <= WP && nsplit >= 1, "delta_tail: sizes must be positive");
+  EI_REQUIRE(J >= 2 && J <= kMaxTaps, "delta_tail: taps must lie between 2 and 32");
+  const size_t total = static_cast<size_t>(N) * C;
+  const size_t ss = static_cast<size_t>(split_stride);
+  if (in_dtype == EI_F32)
+    delta_tail_kernel<float><<<grid_for(total), kThreads, 0, stream>>>(
+        static_cast<const float*>(proj), nsplit, ss, WP, J, state,
+        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
+        seq_slot, seq_start, seq_count, total, C);
+  else if (in_dtype == EI_BF16)
+    delta_tail_kernel<bf16_t><<<grid_for(total), kThreads, 0, stream>>>(
+        static_cast<const bf16_t*>(proj), nsplit, ss, WP, J, state,
+        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
+        seq_slot, seq_start, seq_count, total, C);
+  else
+    EI_REQUIRE(false, "delta_tail: unknown dtype");
+  EI_LAUNCH_CHECK();
+}
+
+// conv [N, 2 G D + H DV] float32; proj as above with the beta and decay projections (H
+// columns each) at beta_col and decay_col; o_raw [N, H DV] float32.  n_seqs blocks walk
+// seq_count rows each from seq_row0.
+extern "C" int ei_delta_rule(const float* conv, const void* proj, int in_dtype, int nsplit,
+                             long long split_stride, int WP, int beta_col, int decay_col,
+                             const float* a_log, const float* dt_bias, float* state,
+                             long long state_stride, const int32_t* seq_slot,
+                             const int32_t* seq_count, const int32_t* seq_row0, float* o_raw,
+                             int n_seqs, int H, int G, int D, int DV, float q_scale,
+                             float unit_eps, hipStream_t stream) {
+  EI_REQUIRE(conv && proj && a_log && dt_bias && state && seq_slot && seq_count && seq_row0 && o_raw,
+             "delta_rule: null pointer");
+  EI_REQUIRE(n_seqs > 0 && H > 0 && G > 0 && H % G == 0 && DV > 0, "delta_rule: bad head counts");
+  EI_REQUIRE(D >= 1 && D <= 256, "delta_rule: the key size must lie between 1 and 256");
+  EI_REQUIRE(beta_col >= 0 && decay_col >= 0 && beta_col + H <= WP && decay_col + H <= WP,
+             "delta_rule: projection columns outside the row");
+  const int L = lanes_a_column(D);
+  const int CB = kThreads / L;
+  const int C = 2 * G * D + H * DV;
+  EI_REQUIRE(H <= 65535 && (DV + CB - 1) / CB <= 65535, "delta_rule: too many heads or columns");
+  dim3 grid(n_seqs, H, (DV + CB - 1) / CB);
+  const size_t ss = static_cast<size_t>(split_stride);
+#define EI_DELTA(TI, LL)                                                                        \
+  delta_rule_kernel<TI, LL><<<grid, kThreads, 0, stream>>>(                                     \
+      conv, C, static_cast<const TI*>(proj), nsplit, ss, WP, beta_col, decay_col, a_log, dt_bias, \
+      state, static_cast<size_t>(state_stride), seq_slot, seq_count, seq_row0, o_raw, H, G, D,  \
+      DV, q_scale, unit_eps)
+#define EI_DELTA_L(TI)                       \
+  do {                                       \
+    if (L == 1) EI_DELTA(TI, 1);             \
+    else if (L == 2) EI_DELTA(TI, 2);        \
+    else if (L == 4) EI_DELTA(TI, 4);        \
+    else if (L == 8) EI_DELTA(TI, 8);        \
+    else if (L == 16) EI_DELTA(TI, 16);      \
+    else EI_DELTA(TI, 32);                   \
+  } while (0)
+  if (in_dtype == EI_F32) EI_DELTA_L(float);
+  else if (in_dtype == EI_BF16) EI_DELTA_L(bf16_t);
+  else EI_REQUIRE(false, "delta_rule: unknown dtype");
+#undef EI_DELTA_L
+#undef EI_DELTA
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_delta_out(const float* o_raw, const void* proj, int in_dtype, int nsplit,
+                            long long split_stride, int WP, int gate_col, const float* norm_w,
+                            float eps, const int32_t* row_seq, void* out, int out_dtype, int N,
+                            int H, int DV, hipStream_t stream) {
+  EI_REQUIRE(o_raw && proj && norm_w && row_seq && out, "delta_out: null pointer");
+  EI_REQUIRE(N > 0 && H > 0 && DV > 0 && nsplit >= 1, "delta_out: sizes must be positive");
+  EI_REQUIRE(gate_col >= 0 && gate_col + H * DV <= WP, "delta_out: gate columns outside the row");
+  EI_REQUIRE(eps > 0.f, "delta_out: eps must be positive");
+  const long long items = static_cast<long long>(N) * H;
+  const long long blocks = (items * EI_WAVE + kThreads - 1) / kThreads;
+  EI_REQUIRE(blocks < (1ll << 31), "delta_out: too many rows");
+  const size_t ss = static_cast<size_t>(split_stride);
+#define EI_DOUT(TI, TO)                                                                      \
+  delta_out_kernel<TI, TO><<<static_cast<unsigned>(blocks), kThreads, 0, stream>>>(          \
+      o_raw, static_cast<const TI*>(proj), nsplit, ss, WP, gate_col, norm_w, eps, row_seq,   \
+      static_cast<TO*>(out), items, H, DV)
+  if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_DOUT(float, float);
+  else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_DOUT(float, bf16_t);
+  else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_DOUT(bf16_t, bf16_t);
+  else EI_REQUIRE(false, "delta_out: unsupported dtype combination");
+#undef EI_DOUT
+  EI_LAUNCH_CHECK();
+}

@@ -31,19 +31,42 @@ _SIGNATURES = {
                       c_void_p],
         "ei_sum_slices": [c_void_p, c_int, c_longlong, c_void_p, c_longlong, c_void_p],
         "ei_bias_rows": [c_void_p, c_void_p, c_longlong, c_int, c_int, c_void_p],
+        "ei_norm_add": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_float, c_void_p,
+                        c_int, c_int, c_int, c_void_p],
+        "ei_cast_rows": [c_void_p, c_void_p, c_int, c_longlong, c_void_p],
+        "ei_activation": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_longlong, c_int,
+                          c_void_p],
     },
     "rope_store": {
         "ei_qk_norm_rope_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_float,
                                   c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                   c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p],
+        "ei_projection_norm_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
+                                     c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                     c_int, c_void_p],
+    },
+    "delta_rule": {
+        "ei_delta_conv": [c_void_p, c_int, c_int, c_longlong, c_int, c_void_p, c_int, c_void_p,
+                          c_longlong, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_int, c_void_p],
+        "ei_delta_tail": [c_void_p, c_int, c_int, c_longlong, c_int, c_int, c_void_p, c_longlong,
+                          c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                          c_int, c_void_p],
+        "ei_delta_rule": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_int, c_int, c_int,
+                          c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p,
+                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
+        "ei_delta_out": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_int, c_int, c_void_p,
+                         c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     },
     "attention_generic": {
         "ei_attn_heads_per_block": [c_int],
         "ei_attn_positions_per_item": [c_int],
         "ei_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                         c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                         c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
+                         c_int, c_void_p],
     },
     "attention_mfma": {
         "ei_attn_decode_mfma_supported": [c_int, c_int],
@@ -264,6 +287,52 @@ def bias_rows(bias: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
     _check(lib, status, "bias_rows")
 
 
+def norm_add(residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float,
+             cast_out: Optional[torch.Tensor] = None) -> None:
+    """residual [R, H] float32 += rmsnorm(sum of delta's slices) * weight; `cast_out` [R, H]
+    (optional) receives the new residual rows in its own type."""
+    lib = library("rowwise")
+    rows, hidden = residual.shape
+    nsplit, stride = _splits(delta, rows, hidden, "delta")
+    if weight.numel() != hidden:
+        raise KernelError(f"norm_add: weight must have {hidden} elements")
+    if cast_out is not None and tuple(cast_out.shape) != (rows, hidden):
+        raise KernelError("norm_add: cast_out must have the residual's shape")
+    status = lib.ei_norm_add(_gpu(residual, "residual", torch.float32), _gpu(delta, "delta"),
+                             _code(delta, "delta"), nsplit, stride,
+                             _gpu(weight, "weight", torch.float32), float(eps),
+                             None if cast_out is None else _gpu(cast_out, "cast_out"),
+                             F32 if cast_out is None else _code(cast_out, "cast_out"), rows, hidden,
+                             _stream())
+    _check(lib, status, "norm_add")
+
+
+def cast_rows(source: torch.Tensor, out: torch.Tensor) -> None:
+    """out = source (float32) in out's type, elementwise."""
+    lib = library("rowwise")
+    if source.numel() != out.numel():
+        raise KernelError("cast_rows: sizes differ")
+    status = lib.ei_cast_rows(_gpu(source, "source", torch.float32), _gpu(out, "out"),
+                              _code(out, "out"), source.numel(), _stream())
+    _check(lib, status, "cast_rows")
+
+
+ACTIVATIONS = {"relu2": 0, "relu": 1, "silu": 2, "gelu_tanh": 3}
+
+
+def activation(x: torch.Tensor, out: torch.Tensor, kind: str) -> None:
+    """out [n, w] = act(x) for x [n, w] or float32 slices [s, n, w] (summed first); kind:
+    "relu2" (relu squared), "relu", "silu", "gelu_tanh"."""
+    lib = library("rowwise")
+    n, width = out.shape
+    nsplit, stride = _splits(x, n, width, "x")
+    if kind not in ACTIVATIONS:
+        raise KernelError(f"activation: unknown kind '{kind}'; known: {sorted(ACTIVATIONS)}")
+    status = lib.ei_activation(_gpu(x, "x"), _code(x, "x"), nsplit, stride, _gpu(out, "out"),
+                               _code(out, "out"), out.numel(), ACTIVATIONS[kind], _stream())
+    _check(lib, status, "activation")
+
+
 def _rotated_width(rope_table, head_dim: int, what: str) -> int:
     """The width of a rotation table [positions, R]: R/2 cosines, then R/2 sines, for the
     pairs (i, i + R/2) of a head's first R <= head_dim elements; the rest pass unrotated."""
@@ -319,21 +388,31 @@ def attention_positions_per_item(group: int) -> int:
 
 def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos, row_seq,
               page_table, out, n_heads, n_kv_heads, head_dim, window=None, scale=None,
-              n_splits=1, part_o=None, part_ml=None) -> None:
-    """Generic causal attention over the paged cache (see attention_generic.hip)."""
+              n_splits=1, part_o=None, part_ml=None, value_dim=None, chunk=None, slopes=None,
+              sinks=None) -> None:
+    """Generic causal attention over the paged cache (see attention_generic.hip).
+    value_dim: head size of the values and of `out` (None: head_dim); chunk: a query sees only
+    the keys of its own block of that many positions; slopes, sinks: float32 [n_heads], the
+    distance term's slope and the softmax's sink of every query head (None: none)."""
     lib = library("attention_generic")
     n = q.shape[0]
-    if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
-        raise KernelError("attention: q and out must be [rows, heads * head_dim]")
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != (n, n_heads * value_dim):
+        raise KernelError("attention: q must be [rows, heads * head_dim] and out "
+                          "[rows, heads * value_dim]")
     expect = (n_kv_heads, PAGE_TOKENS, head_dim)
-    if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != tuple(k_pages.shape):
-        raise KernelError(f"attention: pages must be [*, {expect}]")
+    expect_v = (k_pages.shape[0], n_kv_heads, PAGE_TOKENS, value_dim)
+    if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != expect_v:
+        raise KernelError(f"attention: pages must be [*, {expect}] and {list(expect_v)}")
     if not (q.dtype == k_pages.dtype == v_pages.dtype == out.dtype):
         raise KernelError("attention: q, cache and out dtypes differ")
     if item_seq.numel() < n_items or item_row0.numel() < n_items or item_npos.numel() < n_items:
         raise KernelError("attention: work item arrays shorter than n_items")
+    for name, per_head in (("slopes", slopes), ("sinks", sinks)):
+        if per_head is not None and per_head.numel() != n_heads:
+            raise KernelError(f"attention: {name} must have one value per query head")
     if n_splits > 1:
-        need_o = n * n_heads * n_splits * head_dim
+        need_o = n * n_heads * n_splits * value_dim
         if part_o is None or part_ml is None or part_o.numel() < need_o \
                 or part_ml.numel() < n * n_heads * n_splits * 2:
             raise KernelError("attention: split scratch missing or too small")
@@ -347,8 +426,49 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
         page_table.shape[-1], _gpu(out, "out"),
         None if part_o is None else _gpu(part_o, "part_o", torch.float32),
         None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
-        n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, _stream())
+        n_kv_heads, head_dim, value_dim, int(window or 0), int(chunk or 0),
+        None if slopes is None else _gpu(slopes, "slopes", torch.float32),
+        None if sinks is None else _gpu(sinks, "sinks", torch.float32), float(scale), n_splits,
+        _stream())
     _check(lib, status, "attention")
+
+
+def projection_norm_store(qkv, q_norm_w, k_norm_w, eps, row_pos, row_seq, page_table, q_out,
+                          k_pages, v_pages, n_heads, n_kv_heads, head_dim, value_dim,
+                          write_cache=True) -> None:
+    """One RMS norm over the whole query projection and one over the whole key projection
+    (weights [heads * head_dim] and [kv heads * head_dim], or None for no norm), no rotation;
+    queries to `q_out`, keys [*, kv heads, 64, head_dim] and values [*, kv heads, 64, value_dim]
+    to their cache pages."""
+    lib = library("rope_store")
+    n = q_out.shape[0]
+    width = n_heads * head_dim + n_kv_heads * (head_dim + value_dim)
+    nsplit, stride = _splits(qkv, n, width, "qkv")
+    if tuple(q_out.shape) != (n, n_heads * head_dim):
+        raise KernelError("projection_norm_store: q_out has the wrong shape")
+    if row_pos.numel() < n or row_seq.numel() < n:
+        raise KernelError("projection_norm_store: row metadata shorter than the rows")
+    if (q_norm_w is None) != (k_norm_w is None):
+        raise KernelError("projection_norm_store: both norm weights or neither")
+    if q_norm_w is not None and (q_norm_w.numel() != n_heads * head_dim
+                                 or k_norm_w.numel() != n_kv_heads * head_dim):
+        raise KernelError("projection_norm_store: norm weights must be as wide as the projections")
+    if write_cache:
+        if tuple(k_pages.shape[1:]) != (n_kv_heads, PAGE_TOKENS, head_dim) or \
+                tuple(v_pages.shape) != (k_pages.shape[0], n_kv_heads, PAGE_TOKENS, value_dim):
+            raise KernelError("projection_norm_store: pages have the wrong shape")
+        if k_pages.dtype != q_out.dtype or v_pages.dtype != q_out.dtype:
+            raise KernelError("projection_norm_store: cache and q_out dtypes differ")
+    status = lib.ei_projection_norm_store(
+        _gpu(qkv, "qkv"), _code(qkv, "qkv"), nsplit, stride,
+        None if q_norm_w is None else _gpu(q_norm_w, "q_norm", torch.float32),
+        None if k_norm_w is None else _gpu(k_norm_w, "k_norm", torch.float32), float(eps),
+        _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
+        _gpu(page_table, "page_table", torch.int32), page_table.shape[-1], _gpu(q_out, "q_out"),
+        _gpu(k_pages, "k_pages") if write_cache else None,
+        _gpu(v_pages, "v_pages") if write_cache else None, _code(q_out, "q_out"), n, n_heads,
+        n_kv_heads, head_dim, value_dim, int(write_cache), _stream())
+    _check(lib, status, "projection_norm_store")
 
 
 MFMA_HEAD_DIMS = (64, 128)
@@ -496,6 +616,130 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
         n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, int(waves), int(heads),
         None if longest is None else _gpu(longest, "longest", torch.int32), _stream())
     _check(lib, status, "attention_decode")
+
+
+# -- gated delta rule -----------------------------------------------------------------------
+def delta_state_floats(n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int,
+                       taps: int) -> int:
+    """float32 elements of one sequence's state: S^T of every head [heads, value_dim, key_dim],
+    then the last taps - 1 inputs of every convolved channel [taps - 1, channels], rounded up
+    to a multiple of 4.  (No kernel library is needed to know it.)"""
+    channels = 2 * n_kv_heads * key_dim + n_heads * value_dim
+    return (n_heads * value_dim * key_dim + (taps - 1) * channels + 3) // 4 * 4
+
+
+class DeltaShape:
+    """Sizes of a gated-delta mixer and where its parts lie in a row of its fused projection
+    [q | k | v | beta | decay | gate]."""
+
+    def __init__(self, n_heads, n_kv_heads, key_dim, value_dim, taps):
+        self.n_heads, self.n_kv_heads = int(n_heads), int(n_kv_heads)
+        self.key_dim, self.value_dim, self.taps = int(key_dim), int(value_dim), int(taps)
+        self.qk_width = self.n_kv_heads * self.key_dim
+        self.v_width = self.n_heads * self.value_dim
+        self.channels = 2 * self.qk_width + self.v_width          # what the convolution covers
+        self.beta_col = self.channels
+        self.decay_col = self.beta_col + self.n_heads
+        self.gate_col = self.decay_col + self.n_heads
+        self.width = self.gate_col + self.v_width
+        self.tail_offset = self.n_heads * self.value_dim * self.key_dim
+        self.state_floats = delta_state_floats(n_heads, n_kv_heads, key_dim, value_dim, taps)
+
+
+def _delta_proj(proj, rows, shape):
+    nsplit, stride = _splits(proj, rows, shape.width, "proj")
+    return _gpu(proj, "proj"), _code(proj, "proj"), nsplit, stride
+
+
+def _delta_state(state, shape):
+    if state.dim() != 2 or state.shape[1] != shape.state_floats:
+        raise KernelError(f"delta: the state must be [slots, {shape.state_floats}], "
+                          f"got {list(state.shape)}")
+    return _gpu(state, "state", torch.float32)
+
+
+def delta_conv(proj, conv_w, state, shape: DeltaShape, row_pos, row_seq, seq_slot, seq_start,
+               out) -> None:
+    """out [rows, channels] float32 = silu(causal convolution) of the q, k, v columns of
+    `proj` ([rows, width] or float32 slices of it); conv_w float32 [channels, taps]; inputs
+    from before this step come from the sequences' tails in `state` [slots, state_floats]."""
+    lib = library("delta_rule")
+    rows = out.shape[0]
+    if tuple(out.shape) != (rows, shape.channels) or tuple(conv_w.shape) != (shape.channels, shape.taps):
+        raise KernelError("delta_conv: out must be [rows, channels] and conv_w [channels, taps]")
+    if row_pos.numel() < rows or row_seq.numel() < rows:
+        raise KernelError("delta_conv: row metadata shorter than the rows")
+    pointer, code, nsplit, stride = _delta_proj(proj, rows, shape)
+    status = lib.ei_delta_conv(pointer, code, nsplit, stride, shape.width,
+                               _gpu(conv_w, "conv_w", torch.float32), shape.taps,
+                               _delta_state(state, shape), shape.state_floats, shape.tail_offset,
+                               _gpu(row_pos, "row_pos", torch.int32),
+                               _gpu(row_seq, "row_seq", torch.int32),
+                               _gpu(seq_slot, "seq_slot", torch.int32),
+                               _gpu(seq_start, "seq_start", torch.int32),
+                               _gpu(out, "out", torch.float32), rows, shape.channels, _stream())
+    _check(lib, status, "delta_conv")
+
+
+def delta_tail(proj, state, shape: DeltaShape, rows, row_pos, row_seq, seq_slot, seq_start,
+               seq_count) -> None:
+    """The sequences' tails in `state` become the last taps - 1 inputs after this step."""
+    if shape.taps < 2:
+        return
+    lib = library("delta_rule")
+    pointer, code, nsplit, stride = _delta_proj(proj, rows, shape)
+    status = lib.ei_delta_tail(pointer, code, nsplit, stride, shape.width, shape.taps,
+                               _delta_state(state, shape), shape.state_floats, shape.tail_offset,
+                               _gpu(row_pos, "row_pos", torch.int32),
+                               _gpu(row_seq, "row_seq", torch.int32),
+                               _gpu(seq_slot, "seq_slot", torch.int32),
+                               _gpu(seq_start, "seq_start", torch.int32),
+                               _gpu(seq_count, "seq_count", torch.int32), rows, shape.channels,
+                               _stream())
+    _check(lib, status, "delta_tail")
+
+
+def delta_rule(conv, proj, a_log, dt_bias, state, shape: DeltaShape, seq_slot, seq_count,
+               seq_row0, o_raw, q_scale: float, unit_eps: float) -> None:
+    """The recurrence over every sequence's rows of this step, in order; reads and writes S in
+    `state`; o_raw [rows, heads * value_dim] float32 receives S^T q of every row."""
+    lib = library("delta_rule")
+    rows = conv.shape[0]
+    n_seqs = seq_count.numel()
+    if tuple(conv.shape) != (rows, shape.channels) or tuple(o_raw.shape) != (rows, shape.v_width):
+        raise KernelError("delta_rule: conv must be [rows, channels] and o_raw [rows, heads * value_dim]")
+    if a_log.numel() != shape.n_heads or dt_bias.numel() != shape.n_heads:
+        raise KernelError("delta_rule: one decay rate and bias per head")
+    if seq_slot.numel() < n_seqs or seq_row0.numel() < n_seqs:
+        raise KernelError("delta_rule: sequence metadata shorter than the sequences")
+    pointer, code, nsplit, stride = _delta_proj(proj, rows, shape)
+    status = lib.ei_delta_rule(_gpu(conv, "conv", torch.float32), pointer, code, nsplit, stride,
+                               shape.width, shape.beta_col, shape.decay_col,
+                               _gpu(a_log, "a_log", torch.float32),
+                               _gpu(dt_bias, "dt_bias", torch.float32), _delta_state(state, shape),
+                               shape.state_floats, _gpu(seq_slot, "seq_slot", torch.int32),
+                               _gpu(seq_count, "seq_count", torch.int32),
+                               _gpu(seq_row0, "seq_row0", torch.int32),
+                               _gpu(o_raw, "o_raw", torch.float32), n_seqs, shape.n_heads,
+                               shape.n_kv_heads, shape.key_dim, shape.value_dim, float(q_scale),
+                               float(unit_eps), _stream())
+    _check(lib, status, "delta_rule")
+
+
+def delta_out(o_raw, proj, norm_w, eps, shape: DeltaShape, row_seq, out) -> None:
+    """out [rows, heads * value_dim] = o / sqrt(mean(o^2) + eps) * norm_w * silu(gate) per head."""
+    lib = library("delta_rule")
+    rows = o_raw.shape[0]
+    if tuple(o_raw.shape) != (rows, shape.v_width) or tuple(out.shape) != tuple(o_raw.shape):
+        raise KernelError("delta_out: o_raw and out must be [rows, heads * value_dim]")
+    if norm_w.numel() != shape.value_dim:
+        raise KernelError("delta_out: the norm weight must have value_dim elements")
+    pointer, code, nsplit, stride = _delta_proj(proj, rows, shape)
+    status = lib.ei_delta_out(_gpu(o_raw, "o_raw", torch.float32), pointer, code, nsplit, stride,
+                              shape.width, shape.gate_col, _gpu(norm_w, "norm_w", torch.float32),
+                              float(eps), _gpu(row_seq, "row_seq", torch.int32), _gpu(out, "out"),
+                              _code(out, "out"), rows, shape.n_heads, shape.value_dim, _stream())
+    _check(lib, status, "delta_out")
 
 
 def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:

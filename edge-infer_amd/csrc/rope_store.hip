@@ -349,3 +349,100 @@ extern "C" int ei_qk_norm_rope_store(
 #undef EI_ROPE_LAUNCH
   EI_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------
+// Queries and keys normed over the whole projection (one RMS norm over all heads of q, one
+// over all heads of k, weights of those widths; or no norm), no rotation, and values whose
+// head size may differ from the keys'.  One block a row; sums in float32, one rounding.
+namespace {
+
+template <typename TI, typename TO>
+__global__ void projection_norm_store_kernel(
+    const TI* __restrict__ qkv, int nsplit, size_t split_stride, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, float eps, const int32_t* __restrict__ row_pos,
+    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
+    TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages, int nq, int nkv,
+    int D, int DV, int write_cache) {
+  extern __shared__ float row_values[];     // the row's q, k and v sums
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  const int seq = row_seq[row];
+  if (seq < 0) return;                      // padding row of a fixed-size batch
+  const int QW = nq * D, KW = nkv * D, VW = nkv * DV, W = QW + KW + VW;
+  const TI* src = qkv + static_cast<size_t>(row) * W;
+  float q_sq = 0.f, k_sq = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float x = 0.f;
+    for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TI>(src[s * split_stride + i]);
+    row_values[i] = x;
+    if (i < QW) q_sq += x * x;
+    else if (i < QW + KW) k_sq += x * x;
+  }
+  const float q_total = ei::block_sum(q_sq, scratch);
+  const float k_total = ei::block_sum(k_sq, scratch);
+  const float q_inv = q_norm_w ? 1.0f / sqrtf(q_total / static_cast<float>(QW) + eps) : 1.f;
+  const float k_inv = k_norm_w ? 1.0f / sqrtf(k_total / static_cast<float>(KW) + eps) : 1.f;
+  for (int i = threadIdx.x; i < QW; i += blockDim.x) {
+    const float y = q_norm_w ? (row_values[i] * q_inv) * q_norm_w[i] : row_values[i];
+    q_out[static_cast<size_t>(row) * QW + i] = ei::from_f32<TO>(y);
+  }
+  if (!write_cache) return;
+  const int pos = row_pos[row];
+  const int phys = page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE];
+  if (phys < 0) return;
+  const int in_page = pos % EI_PAGE;
+  for (int i = threadIdx.x; i < KW; i += blockDim.x) {
+    const int head = i / D, d = i % D;
+    const float x = row_values[QW + i];
+    const float y = k_norm_w ? (x * k_inv) * k_norm_w[i] : x;
+    k_pages[((static_cast<size_t>(phys) * nkv + head) * EI_PAGE + in_page) * D + d] =
+        ei::from_f32<TO>(y);
+  }
+  for (int i = threadIdx.x; i < VW; i += blockDim.x) {
+    const int head = i / DV, d = i % DV;
+    v_pages[((static_cast<size_t>(phys) * nkv + head) * EI_PAGE + in_page) * DV + d] =
+        ei::from_f32<TO>(row_values[QW + KW + i]);
+  }
+}
+
+}  // namespace
+
+// qkv: [nsplit][N, nq * D + nkv * D + nkv * DV] of in_dtype; q_out: [N, nq * D]; key pages
+// [n_pages, nkv, 64, D], value pages [n_pages, nkv, 64, DV] of out_dtype; q_norm_w [nq * D] and
+// k_norm_w [nkv * D] float32, or both null (no norm).
+extern "C" int ei_projection_norm_store(
+    const void* qkv, int in_dtype, int nsplit, long long split_stride, const float* q_norm_w,
+    const float* k_norm_w, float eps, const int32_t* row_pos, const int32_t* row_seq,
+    const int32_t* page_table, int table_width, void* q_out, void* k_pages, void* v_pages,
+    int out_dtype, int N, int nq, int nkv, int D, int DV, int write_cache, hipStream_t stream) {
+  EI_REQUIRE(N > 0 && nq > 0 && nkv > 0 && D > 0 && DV > 0,
+             "projection_norm_store: sizes must be positive");
+  EI_REQUIRE(qkv && row_pos && row_seq && q_out, "projection_norm_store: null pointer");
+  EI_REQUIRE((q_norm_w == nullptr) == (k_norm_w == nullptr),
+             "projection_norm_store: both norm weights or neither");
+  EI_REQUIRE(!write_cache || (k_pages && v_pages && page_table && table_width > 0),
+             "projection_norm_store: cache pointers missing");
+  EI_REQUIRE(nsplit >= 1, "projection_norm_store: nsplit must be at least 1");
+  const long long width = static_cast<long long>(nq) * D + static_cast<long long>(nkv) * (D + DV);
+  EI_REQUIRE(width * 4 <= 160 * 1024 - 1024, "projection_norm_store: the row does not fit in LDS");
+  const size_t lds = static_cast<size_t>(width) * sizeof(float);
+  const int threads = width >= 2048 ? 512 : 256;
+  const size_t ss = static_cast<size_t>(split_stride);
+#define EI_PNS(TI, TO)                                                                          \
+  do {                                                                                          \
+    if (lds > 64 * 1024)                                                                        \
+      (void)hipFuncSetAttribute(                                                                \
+          reinterpret_cast<const void*>(&projection_norm_store_kernel<TI, TO>),                 \
+          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));                   \
+    projection_norm_store_kernel<TI, TO><<<N, threads, lds, stream>>>(                          \
+        static_cast<const TI*>(qkv), nsplit, ss, q_norm_w, k_norm_w, eps, row_pos, row_seq,     \
+        page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),            \
+        static_cast<TO*>(v_pages), nq, nkv, D, DV, write_cache);                                \
+  } while (0)
+  if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_PNS(float, float);
+  else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_PNS(float, bf16_t);
+  else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_PNS(bf16_t, bf16_t);
+  else EI_REQUIRE(false, "projection_norm_store: unsupported dtype combination");
+#undef EI_PNS
+  EI_LAUNCH_CHECK();
+}

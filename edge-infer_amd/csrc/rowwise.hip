@@ -387,3 +387,131 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
     EI_REQUIRE(false, "swiglu: unsupported dtype combination");
   EI_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------
+// Kernels for blocks whose norm sits on a sublayer's output: residual += rmsnorm(delta) * w.
+namespace {
+
+// One block per row.  x = sum over slices of delta[row]; residual[row] += x * rsqrt(mean(x^2)
+// + eps) * weight; optionally the new residual row is also written in the storage type (what
+// the next sublayer's product reads).
+template <typename TD, typename TO>
+__global__ void norm_add_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                int nsplit, size_t split_stride, const float* __restrict__ weight,
+                                float eps, TO* __restrict__ cast_out, int H) {
+  extern __shared__ float row_values[];
+  __shared__ float scratch[16];
+  const size_t base = static_cast<size_t>(blockIdx.x) * H;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const TD* d = delta + base + i;
+    float x = 0.f;
+    for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TD>(d[s * split_stride]);
+    row_values[i] = x;
+    sum += x * x;
+  }
+  const float total = ei::block_sum(sum, scratch);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(H) + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float y = residual[base + i] + (row_values[i] * inv) * weight[i];
+    residual[base + i] = y;
+    if (cast_out) cast_out[base + i] = ei::from_f32<TO>(y);
+  }
+}
+
+template <typename TO>
+__global__ void cast_rows_kernel(const float* __restrict__ in, TO* __restrict__ out, size_t n) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = start; i < n; i += step) out[i] = ei::from_f32<TO>(in[i]);
+}
+
+// activation kinds of the C interface
+constexpr int kRelu2 = 0, kRelu = 1, kSilu = 2, kGeluTanh = 3;
+
+__device__ __forceinline__ float activate(float x, int kind) {
+  if (kind == kRelu2) {
+    const float r = fmaxf(x, 0.f);
+    return r * r;
+  }
+  if (kind == kRelu) return fmaxf(x, 0.f);
+  if (kind == kSilu) return x / (1.0f + expf(-x));
+  // 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))
+  return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+
+// out = act(sum over slices of in), elementwise.
+template <typename TI, typename TO>
+__global__ void activation_kernel(const TI* __restrict__ in, int nsplit, size_t split_stride,
+                                  TO* __restrict__ out, size_t n, int kind) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = start; i < n; i += step) {
+    float x = 0.f;
+    for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TI>(in[s * split_stride + i]);
+    out[i] = ei::from_f32<TO>(activate(x, kind));
+  }
+}
+
+}  // namespace
+
+// residual [N, H] float32 += rmsnorm(sum of delta slices) * weight; cast_out (or null): the
+// new residual rows in out_dtype.
+extern "C" int ei_norm_add(float* residual, const void* delta, int delta_dtype, int nsplit,
+                           long long split_stride, const float* weight, float eps, void* cast_out,
+                           int out_dtype, int N, int H, hipStream_t stream) {
+  EI_REQUIRE(N > 0 && H > 0, "norm_add: sizes must be positive");
+  EI_REQUIRE(H <= 16384, "norm_add: width above 16384 is not supported");
+  EI_REQUIRE(residual && delta && weight && nsplit >= 1, "norm_add: bad arguments");
+  EI_REQUIRE(eps > 0.f, "norm_add: eps must be positive");
+  const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
+  const size_t lds = static_cast<size_t>(H) * sizeof(float);
+  const size_t ss = static_cast<size_t>(split_stride);
+#define EI_NORM_ADD(TD, TO)                                                                      \
+  norm_add_kernel<TD, TO><<<N, threads, lds, stream>>>(residual, static_cast<const TD*>(delta),  \
+                                                       nsplit, ss, weight, eps,                  \
+                                                       static_cast<TO*>(cast_out), H)
+  if (delta_dtype == EI_F32 && (out_dtype == EI_F32 || !cast_out)) EI_NORM_ADD(float, float);
+  else if (delta_dtype == EI_F32 && out_dtype == EI_BF16) EI_NORM_ADD(float, bf16_t);
+  else if (delta_dtype == EI_BF16 && (out_dtype == EI_BF16 || !cast_out)) EI_NORM_ADD(bf16_t, bf16_t);
+  else EI_REQUIRE(false, "norm_add: unsupported dtype combination");
+#undef EI_NORM_ADD
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_cast_rows(const float* in, void* out, int out_dtype, long long n,
+                            hipStream_t stream) {
+  EI_REQUIRE(in && out && n > 0, "cast_rows: bad arguments");
+  const int threads = 256;
+  long long blocks = (n + threads - 1) / threads;
+  if (blocks > ei_compute_units() * 16) blocks = ei_compute_units() * 16;
+  if (out_dtype == EI_BF16)
+    cast_rows_kernel<bf16_t><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+        in, static_cast<bf16_t*>(out), static_cast<size_t>(n));
+  else if (out_dtype == EI_F32)
+    cast_rows_kernel<float><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+        in, static_cast<float*>(out), static_cast<size_t>(n));
+  else
+    EI_REQUIRE(false, "cast_rows: unknown dtype");
+  EI_LAUNCH_CHECK();
+}
+
+// out [n] = act(sum of `nsplit` slices of in); kind 0: relu(x)^2, 1: relu, 2: silu, 3: tanh gelu.
+extern "C" int ei_activation(const void* in, int in_dtype, int nsplit, long long split_stride,
+                             void* out, int out_dtype, long long n, int kind, hipStream_t stream) {
+  EI_REQUIRE(in && out && n > 0 && nsplit >= 1, "activation: bad arguments");
+  EI_REQUIRE(kind >= 0 && kind <= 3, "activation: unknown kind");
+  const int threads = 256;
+  long long blocks = (n + threads - 1) / threads;
+  if (blocks > ei_compute_units() * 32) blocks = ei_compute_units() * 32;
+  const size_t ss = static_cast<size_t>(split_stride);
+#define EI_ACT(TI, TO)                                                                         \
+  activation_kernel<TI, TO><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(            \
+      static_cast<const TI*>(in), nsplit, ss, static_cast<TO*>(out), static_cast<size_t>(n), kind)
+  if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_ACT(float, float);
+  else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_ACT(float, bf16_t);
+  else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_ACT(bf16_t, bf16_t);
+  else EI_REQUIRE(false, "activation: unsupported dtype combination");
+#undef EI_ACT
+  EI_LAUNCH_CHECK();
+}

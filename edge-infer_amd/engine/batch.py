@@ -8,7 +8,8 @@ in one int32 buffer of named sections:
   tokens[N] row_pos[N] row_seq[N]      per row: token id, position, index of its sequence
   want_rows[W]                         rows whose logits are wanted
   seq_slot[B] seq_start[B] seq_count[B]  per sequence: cache slot (its row in every state
-                                       table), tokens held before the step, tokens brought
+  seq_row0[B]                          table), tokens held before the step, tokens brought,
+                                       the first of its packed rows
   pages<g>[B, width]                   per key/value group: logical page -> physical page
   ...                                  whatever the model's parts plan for themselves
 
@@ -84,6 +85,9 @@ class StepPlan:
         self.seq_slot = np.full(self.n_seqs, spare_slot, dtype=np.int32)
         self.seq_start = np.zeros(self.n_seqs, dtype=np.int32)
         self.seq_count = np.zeros(self.n_seqs, dtype=np.int32)
+        self.seq_row0 = np.zeros(self.n_seqs, dtype=np.int32)
+        self.seq_row0[:len(seqs)] = np.fromiter((seq.row0 for seq in seqs), dtype=np.int32,
+                                                count=len(seqs))
         want_rows: List[int] = []
         if self.decode:                  # one row a sequence: whole arrays at once
             live = len(seqs)
@@ -136,7 +140,8 @@ class StepPlan:
         out = [("longest", np.asarray([self.max_context], dtype=np.int32)),
                ("tokens", self.tokens), ("row_pos", self.row_pos), ("row_seq", self.row_seq),
                ("want_rows", self.want_rows), ("seq_slot", self.seq_slot),
-               ("seq_start", self.seq_start), ("seq_count", self.seq_count)]
+               ("seq_start", self.seq_start), ("seq_count", self.seq_count),
+               ("seq_row0", self.seq_row0)]
         for index, table in enumerate(page_tables):
             out.append((f"pages{index}", table.reshape(-1)))
         for name, array in self.extra.items():
@@ -234,6 +239,7 @@ class DeviceMeta:
     seq_slot = property(lambda self: self.section("seq_slot"))
     seq_start = property(lambda self: self.section("seq_start"))
     seq_count = property(lambda self: self.section("seq_count"))
+    seq_row0 = property(lambda self: self.section("seq_row0"))
 
     def page_table(self, group: int) -> torch.Tensor:
         return self.section(f"pages{group}").view(self.n_seqs, self._table_widths[group])

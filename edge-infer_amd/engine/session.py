@@ -189,7 +189,7 @@ class Session:
             self._sampler = Sampler(self.device)
         spec = self.model.spec
         if stop_ids is None:
-            stop_ids = (spec.eos_token_id,)
+            stop_ids = () if spec.eos_token_id is None else (spec.eos_token_id,)
         if first_stream is None:
             first_stream = self._streams_used
             self._streams_used += len(prompts)

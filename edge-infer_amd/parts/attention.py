@@ -7,6 +7,13 @@ runtime/include/execution/decoder.hpp:121-158.  Three separate checkpoint matric
 become one [Q + 2 KV, H] matrix when the part is built: each output element is
 still the same dot product.  Each projection may have a bias
 (runtime/include/models/qwen3_model.hpp:386-395: taken if the checkpoint holds it).
+
+Options of the spec beyond that decoder (any of them sends the mixer down the generic
+float32-arithmetic kernels): values narrower or wider than keys (`value_dim`), one RMS norm
+over the whole q and the whole k projection instead of one per head (`qk_norm_scope =
+"projection"`), visibility in blocks of `chunk` positions counted from the sequence's start,
+a distance term slope_h (i - j) taken off the score with slope_h = 2^(-r (h + 1) / heads)
+(`distance_slope_range` = r), and a learned `sink` per head in the softmax's denominator.
 """
 from __future__ import annotations
 
@@ -64,28 +71,38 @@ class Attention:
         params = {
             "q_proj.weight": ParamSpec((spec.q_width, hidden)),
             "k_proj.weight": ParamSpec((spec.kv_width, hidden)),
-            "v_proj.weight": ParamSpec((spec.kv_width, hidden)),
-            "o_proj.weight": ParamSpec((hidden, spec.q_width)),
-            "q_proj.bias": ParamSpec((spec.q_width,), optional=True),
-            "k_proj.bias": ParamSpec((spec.kv_width,), optional=True),
-            "v_proj.bias": ParamSpec((spec.kv_width,), optional=True),
+            "v_proj.weight": ParamSpec((spec.v_width, hidden)),
+            "o_proj.weight": ParamSpec((hidden, spec.out_width)),
             "o_proj.bias": ParamSpec((hidden,), optional=True),
         }
+        if spec.qkv_bias is not False:
+            required = spec.qkv_bias is True
+            params["q_proj.bias"] = ParamSpec((spec.q_width,), optional=not required)
+            params["k_proj.bias"] = ParamSpec((spec.kv_width,), optional=not required)
+            params["v_proj.bias"] = ParamSpec((spec.v_width,), optional=not required)
         if spec.qk_norm:
-            params["q_norm.weight"] = ParamSpec((spec.head_dim,), init="norm")
-            params["k_norm.weight"] = ParamSpec((spec.head_dim,), init="norm")
+            whole = spec.qk_norm_scope == "projection"
+            params["q_norm.weight"] = ParamSpec((spec.q_width if whole else spec.head_dim,),
+                                                init="norm")
+            params["k_norm.weight"] = ParamSpec((spec.kv_width if whole else spec.head_dim,),
+                                                init="norm")
+        if spec.sink:
+            params["sink"] = ParamSpec((spec.n_heads,), init="uniform", low=-1.0, high=1.0)
         return params
 
     @classmethod
     def cache_request(cls, spec):
-        return KVRequest(n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window)
+        return KVRequest(n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window,
+                         value_dim=None if spec.v_dim == spec.head_dim else spec.v_dim,
+                         chunk=spec.chunk)
 
     @classmethod
     def kernel_libraries(cls, spec, dtype):
         """What this part will run, so that a model can have it compiled ahead of its first
         step."""
         group = spec.n_heads // max(1, spec.n_kv_heads)
-        fast = dtype == torch.bfloat16 and lib.attention_decode_mfma_supported(spec.head_dim, group)
+        fast = (dtype == torch.bfloat16 and not spec.extended
+                and lib.attention_decode_mfma_supported(spec.head_dim, group))
         return ("rope_store", "attention_mfma" if fast else "attention_generic",
                 *Linear.kernel_libraries(dtype))
 
@@ -93,11 +110,28 @@ class Attention:
     def check(cls, spec):
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("attention: n_heads must be a multiple of n_kv_heads")
-        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
-            raise ValueError("attention: head_dim must be a multiple of 16 between 16 and 256, "
-                             f"got {spec.head_dim}")
+        if spec.qk_norm_scope not in ("head", "projection"):
+            raise ValueError(f"attention: unknown qk_norm_scope '{spec.qk_norm_scope}'")
+        whole = spec.qk_norm_scope == "projection" or not spec.qk_norm
+        if whole and spec.position.kind == "none":
+            # the store kernel without a rotation takes any sizes the attention kernel takes
+            if not (1 <= spec.head_dim <= 256 and 1 <= spec.v_dim <= 256):
+                raise ValueError("attention: key and value head sizes must lie in 1..256, got "
+                                 f"{spec.head_dim} and {spec.v_dim}")
+        else:
+            if spec.qk_norm_scope == "projection" and spec.qk_norm:
+                raise ValueError("attention: a norm over the whole projection is implemented "
+                                 "only without a rotation")
+            if spec.v_dim != spec.head_dim:
+                raise ValueError("attention: values of another width than the keys are "
+                                 "implemented only without a rotation and per-head norms")
+            if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
+                raise ValueError("attention: head_dim must be a multiple of 16 between 16 and "
+                                 f"256, got {spec.head_dim}")
         if spec.window is not None and spec.window < 1:
             raise ValueError("attention: a window must be at least 1")
+        if spec.chunk is not None and spec.chunk < 1:
+            raise ValueError("attention: a chunk must hold at least one position")
 
     def __init__(self, spec, hidden, params, dtype, device, positions):
         self.check(spec)
@@ -122,9 +156,19 @@ class Attention:
         self.position = positions(spec.position)   # shared table object
         self.group = spec.n_heads // spec.n_kv_heads
         self.scale = spec.scale if spec.scale is not None else spec.head_dim ** -0.5
-        # the matrix-core kernels take bfloat16 with head sizes 64 and 128; every other
-        # case runs the generic kernel
-        self.matrix_cores = (dtype == torch.bfloat16 and
+        # without a rotation and without per-head norms, one kernel norms (or not) and stores
+        self.whole_store = (spec.position.kind == "none"
+                            and (spec.qk_norm_scope == "projection" or not spec.qk_norm))
+        self.slopes = self.sinks = None
+        if spec.distance_slope_range is not None:
+            exponent = -float(spec.distance_slope_range) * torch.arange(
+                1, spec.n_heads + 1, dtype=torch.float64) / spec.n_heads
+            self.slopes = torch.pow(2.0, exponent).to(device=device, dtype=torch.float32).contiguous()
+        if spec.sink:
+            self.sinks = params["sink"].to(device=device, dtype=torch.float32).contiguous()
+        # the matrix-core kernels take bfloat16 with head sizes 64 and 128 and none of the
+        # options beyond rotary, windowed attention; every other case runs the generic kernel
+        self.matrix_cores = (dtype == torch.bfloat16 and not spec.extended and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
         self.compute_units = lib.compute_units(device)     # the chip's size, for launch plans
         self._decode_launches = {}     # (sequences, pages of context) -> decode_launch's answer
@@ -201,6 +245,8 @@ class Attention:
         unit, never more than there are pages."""
         if self.spec.window is not None:
             context = min(context, self.spec.window + PAGE_TOKENS - 1)
+        if self.spec.chunk is not None:
+            context = min(context, self.spec.chunk + PAGE_TOKENS - 1)
         pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
         n_kv_heads = self.spec.n_kv_heads
         units = self.compute_units
@@ -262,18 +308,25 @@ class Attention:
             # the decode kernel norms, rotates and stores for its rows itself: one launch less
             q = lib.DecodeProjection(qkv, self.q_norm, self.k_norm, spec.qk_norm_eps,
                                      self.position.table, entry.writes_cache)
+        elif self.whole_store:
+            q = ctx.buffer("attn.q", (n, spec.q_width))
+            lib.projection_norm_store(
+                qkv, self.q_norm, self.k_norm, spec.qk_norm_eps, meta.row_pos, meta.row_seq,
+                page_table, q, k_pages, v_pages, spec.n_heads, spec.n_kv_heads, spec.head_dim,
+                spec.v_dim, write_cache=entry.writes_cache)
         else:
             q = ctx.buffer("attn.q", (n, spec.q_width))
             lib.qk_norm_rope_store(
                 qkv, self.q_norm, self.k_norm, spec.qk_norm_eps, self.position.table,
                 meta.row_pos, meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads,
                 spec.n_kv_heads, spec.head_dim, write_cache=entry.writes_cache)
-        out = ctx.buffer("attn.out", (n, spec.q_width))
+        out = ctx.buffer("attn.out", (n, spec.out_width))
+        more = dict(value_dim=spec.v_dim, chunk=spec.chunk, slopes=self.slopes, sinks=self.sinks)
         part_o = part_ml = None
         if ctx.decode:
             splits, waves, heads = self._decode_launch_for(ctx.n_seqs, ctx.context_bound)
             if splits > 1:
-                part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
+                part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.v_dim,),
                                     torch.float32)
                 part_ml = ctx.buffer("attn.part_ml", (n * spec.n_heads * splits * 2,),
                                      torch.float32)
@@ -288,7 +341,8 @@ class Attention:
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
                               spec.n_kv_heads, spec.head_dim, window=spec.window,
-                              scale=self.scale, n_splits=splits, part_o=part_o, part_ml=part_ml)
+                              scale=self.scale, n_splits=splits, part_o=part_o, part_ml=part_ml,
+                              **more)
         else:
             key_ways = self.prefill_key_ways([seq.count for seq in ctx.sequences])
             section = self._items_section(key_ways)
@@ -309,7 +363,7 @@ class Attention:
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
                               spec.n_kv_heads, spec.head_dim, window=spec.window,
-                              scale=self.scale)
+                              scale=self.scale, **more)
         ctx.release(qkv, None if isinstance(q, lib.DecodeProjection) else q, part_o, part_ml)
         delta = self.o.forward(ctx, out, "attn.o")
         ctx.release(out)

@@ -26,11 +26,13 @@ import torch
 class KVRequest:
     """Keys and values for every position (or the last `window`) of a sequence: pages
     [kv_heads, 64, head_dim] of keys and [kv_heads, 64, value_dim] of values (`value_dim`
-    None: as wide as the keys)."""
+    None: as wide as the keys).  `chunk`: a query sees only keys of its own block of that many
+    positions, so pages that lie wholly before the block of the next position are given back."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
+    chunk: Optional[int] = None
 
 
 @dataclass(frozen=True)

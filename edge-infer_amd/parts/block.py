@@ -1,6 +1,9 @@
 """Arrangements of norm, mixer and feed-forward in one layer."""
 from __future__ import annotations
 
+import torch
+
+from ..csrc import lib
 from .registry import lookup
 
 
@@ -69,3 +72,106 @@ class PreNormBlock:
         out = self.ffn.forward(ctx, h2)
         ctx.release(h2)
         return out
+
+
+class OutputNormBlock:
+    """x += norm1(mixer(x)); x += norm2(feed_forward(x)): the sublayers read the residual
+    stream itself and each norm sits on its sublayer's output.  A layer may have no
+    feed-forward (then it has no second norm either).
+
+    The stream is float32; a sublayer's products read it in the step's storage type.  In
+    float32 that is the stream itself; in bfloat16 the norm kernel that adds a sublayer's
+    output also writes the rounded rows for the next reader (two buffers in turn, since a
+    reader's copy is still live while the next one is written), and only a model's first
+    layer needs a cast kernel of its own.  The block returns no pending delta: everything is
+    added when it returns."""
+
+    capture_safe = True      # nothing of its own besides its parts' kernels and the cast
+    CAST_NOTE = "outnorm.cast"     # ctx.notes: (stream rows in the storage type, index of its buffer)
+
+    def members(self):
+        return tuple(part for part in (self.mixer, self.norm1, self.ffn, self.norm2)
+                     if part is not None)
+
+    @classmethod
+    def _owners(cls, layer_spec):
+        norm_cls = lookup("norm", layer_spec.norm.kind)
+        owners = [("mixer", lookup("mixer", layer_spec.mixer.kind), layer_spec.mixer),
+                  ("norm1", norm_cls, layer_spec.norm)]
+        if layer_spec.feed_forward is not None:
+            owners += [("ffn", lookup("feed_forward", layer_spec.feed_forward.kind),
+                        layer_spec.feed_forward),
+                       ("norm2", norm_cls, layer_spec.norm)]
+        return owners
+
+    @classmethod
+    def parameters(cls, layer_spec, hidden):
+        params = {}
+        for prefix, owner, spec in cls._owners(layer_spec):
+            for name, param in owner.parameters(spec, hidden).items():
+                params[f"{prefix}.{name}"] = param
+        return params
+
+    @classmethod
+    def mixer_spec(cls, layer_spec):
+        return layer_spec.mixer
+
+    @classmethod
+    def kernel_libraries(cls, layer_spec, dtype):
+        names = ["rowwise"]
+        for _, owner, spec in cls._owners(layer_spec):
+            ask = getattr(owner, "kernel_libraries", None)
+            if ask is not None:
+                names.extend(ask(spec, dtype))
+        return tuple(names)
+
+    def __init__(self, layer_spec, hidden, params, dtype, device, positions):
+        def sub(prefix):
+            return {name[len(prefix) + 1:]: tensor for name, tensor in params.items()
+                    if name.startswith(prefix + ".")}
+        norm_cls = lookup("norm", layer_spec.norm.kind)
+        if not hasattr(norm_cls, "norm_add"):
+            raise ValueError(f"norm kind '{layer_spec.norm.kind}' cannot sit on a sublayer's output")
+        self.mixer = lookup("mixer", layer_spec.mixer.kind)(
+            layer_spec.mixer, hidden, sub("mixer"), dtype, device, positions=positions)
+        self.norm1 = norm_cls(layer_spec.norm, hidden, sub("norm1"), dtype, device)
+        self.ffn = self.norm2 = None
+        if layer_spec.feed_forward is not None:
+            self.ffn = lookup("feed_forward", layer_spec.feed_forward.kind)(
+                layer_spec.feed_forward, hidden, sub("ffn"), dtype, device)
+            self.norm2 = norm_cls(layer_spec.norm, hidden, sub("norm2"), dtype, device)
+        self.narrow = dtype != torch.float32
+
+    def _stream_rows(self, ctx, residual):
+        """The stream as the products read it, and which of the two cast buffers holds it."""
+        if not self.narrow:
+            return residual, 0
+        held = ctx.notes.pop(self.CAST_NOTE, None)
+        if held is not None:
+            return held
+        rows = ctx.buffer("outnorm.x0", tuple(residual.shape))
+        lib.cast_rows(residual, rows)
+        return rows, 0
+
+    def forward(self, ctx, residual, pending, entry):
+        if pending is not None:
+            raise ValueError("outnorm: a delta of the block before is still pending; this "
+                             "arrangement follows only blocks that add everything themselves")
+        x, index = self._stream_rows(ctx, residual)
+        a = self.mixer.forward(ctx, x, entry)
+        if self.narrow:
+            ctx.release(x)
+        x = self.norm1.norm_add(ctx, residual, a, f"outnorm.x{1 - index}" if self.narrow else None)
+        ctx.release(a)
+        index = 1 - index
+        if self.ffn is not None:
+            f = self.ffn.forward(ctx, residual if x is None else x)
+            if self.narrow:
+                ctx.release(x)
+            x = self.norm2.norm_add(ctx, residual, f,
+                                    f"outnorm.x{1 - index}" if self.narrow else None)
+            ctx.release(f)
+            index = 1 - index
+        if self.narrow:
+            ctx.notes[self.CAST_NOTE] = (x, index)
+        return None

@@ -1,4 +1,7 @@
-"""Gated feed-forward: down(silu(gate(x)) * up(x)).
+"""Feed-forward parts.  `GatedMLP`: down(silu(gate(x)) * up(x)); `DenseMLP`:
+down(act(up(x))) with act one of relu squared, relu, silu, tanh-gelu.
+
+The gated one:
 
 runtime/include/execution/decoder.hpp:161-166 of the reference; gate and up are
 two checkpoint matrices that become one [2I, H] matrix when the part is built: in strips
@@ -77,6 +80,52 @@ class GatedMLP:
             act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
             lib.swiglu(gate_up, act, self.strip)
             ctx.release(gate_up)
+        out = self.down.forward(ctx, act, "mlp.down")
+        ctx.release(act)
+        return out
+
+
+class DenseMLP:
+    """down(act(up(x))): two matrices and an elementwise activation between them
+    (`spec.activation`: "relu2" = relu(z)^2, "relu", "silu", "gelu_tanh").  The activation
+    kernel sums the float32 slices of a few-rows product while it reads them."""
+
+    @property
+    def capture_safe(self):
+        return self.up.capture_safe and self.down.capture_safe
+
+    @property
+    def capture_rows(self):
+        return min(self.up.capture_rows, self.down.capture_rows)
+
+    @classmethod
+    def kernel_libraries(cls, spec, dtype):
+        return ("rowwise", *Linear.kernel_libraries(dtype))
+
+    @classmethod
+    def parameters(cls, spec, hidden):
+        return {
+            "up_proj.weight": ParamSpec((spec.intermediate_size, hidden)),
+            "down_proj.weight": ParamSpec((hidden, spec.intermediate_size)),
+            "up_proj.bias": ParamSpec((spec.intermediate_size,), optional=True),
+            "down_proj.bias": ParamSpec((hidden,), optional=True),
+        }
+
+    def __init__(self, spec, hidden, params, dtype, device):
+        if spec.activation not in lib.ACTIVATIONS:
+            raise ValueError(f"dense_mlp: activation '{spec.activation}' is not implemented; "
+                             f"known: {sorted(lib.ACTIVATIONS)}")
+        self.spec = spec
+        self.up = Linear(params["up_proj.weight"], dtype, device, bias=params.get("up_proj.bias"))
+        self.down = Linear(params["down_proj.weight"], dtype, device,
+                           bias=params.get("down_proj.bias"))
+
+    def forward(self, ctx, x):
+        n = x.shape[0]
+        up = self.up.forward(ctx, x, "mlp.up")
+        act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
+        lib.activation(up, act, self.spec.activation)
+        ctx.release(up)
         out = self.down.forward(ctx, act, "mlp.down")
         ctx.release(act)
         return out

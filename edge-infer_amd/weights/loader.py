@@ -22,12 +22,16 @@ import torch
 @dataclass(frozen=True)
 class ParamSpec:
     """One parameter a part expects.  `init` chooses the random-weights law:
-    "normal" (N(0, 0.02)) for matrices and tables, "norm" (1 + U(-0.1, 0.1)).
+    "normal" (N(0, scale), scale 0.02 unless given) for matrices and tables, "norm"
+    (1 + U(-0.1, 0.1)), "uniform" (U(low, high)).
     `optional`: taken when the checkpoint holds it, no error when it does not (the
     reference's optional projection biases, runtime/include/models/qwen3_model.hpp:371-403)."""
     shape: Tuple[int, ...]
     init: str = "normal"
     optional: bool = False
+    scale: float = 0.02
+    low: float = 0.0
+    high: float = 1.0
 
 
 @dataclass

@@ -18,10 +18,13 @@ def random_tensor(spec: ParamSpec, generator: torch.Generator, device="cpu",
                   dtype=torch.bfloat16) -> torch.Tensor:
     shape = tuple(spec.shape)
     if spec.init == "normal":
-        value = torch.randn(shape, generator=generator, device=device, dtype=torch.float32) * 0.02
+        value = torch.randn(shape, generator=generator, device=device, dtype=torch.float32) * spec.scale
     elif spec.init == "norm":
         value = 1.0 + (torch.rand(shape, generator=generator, device=device,
                                   dtype=torch.float32) * 0.2 - 0.1)
+    elif spec.init == "uniform":
+        value = spec.low + (spec.high - spec.low) * torch.rand(
+            shape, generator=generator, device=device, dtype=torch.float32)
     else:
         raise ValueError(f"unknown initialisation '{spec.init}'")
     return value.to(dtype)
