@@ -250,6 +250,8 @@ class DecoderModel:
         are planned by the workspace per shape of step: rows, sequences, wanted rows, kind,
         and, for a captured step, the context bound that fixes the parts' launch shapes."""
         workspace = ctx.workspace
+        ctx.notes.clear()      # what the parts note lives for one pass (a step that is captured
+        #                        runs two passes over one context: eagerly, then recorded)
         workspace.start(*workspace_class(ctx))
         try:
             logits = self._forward(ctx)
