@@ -11,7 +11,8 @@
 their caches.  Beyond the reference, a session can serve a batch of prompts
 (`new_session(max_batch=8)`, `session.generate_batch`) and exposes the step function
 (`session.step`).  Model types: "qwen3_bf16" (the reference's name) and
-"qwen3_fp32" for the true 32-bit path.
+"qwen3_fp32" for the true 32-bit path; "tirurax_bf16" and "tirurax_fp32" likewise for
+Tirurax folders.
 
 The reference's procedural wrappers over one implicit session are here too
 (model_bridge.cpp:159-215,274-283): `init_model`, `generate_text_stream`,
@@ -33,7 +34,8 @@ from .engine.session import Session
 from .sampling.params import SamplingParams  # noqa: F401
 from .weights import read_tensors
 
-MODEL_TYPES = {"qwen3_bf16": "bfloat16", "qwen3_fp32": "float32"}
+MODEL_TYPES = {"qwen3_bf16": "bfloat16", "qwen3_fp32": "float32",
+               "tirurax_bf16": "bfloat16", "tirurax_fp32": "float32"}
 DEFAULT_CAPACITY = 4096   # bindings/python/model_bridge.cpp:135-141: min(4096, model limit)
 
 
@@ -66,6 +68,10 @@ class Model:
             raise ValueError("this library runs on the GPU only (device 'cuda')")
         self._device = require_gpu(device or "cuda")
         entry = resolve_architecture(config)
+        family = model_type.rsplit("_", 1)[0]
+        if family not in entry.model_types:
+            raise ValueError(f"model type {model_type!r} names the family '{family}', but the "
+                             f"configuration is a {entry.name} ({'/'.join(entry.model_types)})")
         self.config = entry.config_class.from_dict(config)
         self.decoder = build_model(entry, self.config, weights, dtype, self._device)
         self.model_type = model_type

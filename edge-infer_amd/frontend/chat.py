@@ -20,7 +20,7 @@ import sys
 import time
 from pathlib import Path
 
-MODEL_TYPES = ("qwen3_bf16", "qwen3_fp32")
+MODEL_TYPES = ("qwen3_bf16", "qwen3_fp32", "tirurax_bf16", "tirurax_fp32")
 
 
 def load_tokenizer(model_path):
@@ -141,11 +141,12 @@ class TextStream:
 
 
 def build_parser() -> argparse.ArgumentParser:
-    parser = argparse.ArgumentParser(description="Qwen3 chat / generation on one MI355X")
+    parser = argparse.ArgumentParser(description="chat / generation on one MI355X")
     parser.add_argument("--model_path", type=str, required=True,
                         help="local folder with config.json, safetensors and (for text) tokenizer.json")
     parser.add_argument("--model_type", type=str, default="qwen3_bf16", choices=MODEL_TYPES,
-                        help="qwen3_bf16, or qwen3_fp32 for the true 32-bit path")
+                        help="<family>_bf16, or <family>_fp32 for the true 32-bit path; the "
+                             "family (qwen3, tirurax) must be the one config.json names")
     parser.add_argument("--device", type=str, default="cuda", choices=["cuda"],
                         help="execution device (this library runs on the GPU only)")
     parser.add_argument("--system_prompt", type=str, default="You are a helpful AI assistant.")
@@ -206,13 +207,17 @@ def main(argv=None) -> int:
 
     from ..api import Model
     model = Model.from_pretrained(args.model_path, args.model_type, device=args.device)
-    cfg = model.config
+    cfg, spec = model.config, model.decoder.spec
     print(f"Model Type: {args.model_type}")
-    print(f"Hidden Size: {cfg.hidden_size}")
-    print(f"Num Layers: {cfg.num_hidden_layers}")
-    print(f"Num Attention Heads: {cfg.num_attention_heads}")
-    print(f"Num KV Heads: {cfg.num_key_value_heads}")
-    print(f"Head Dimension: {cfg.head_dim}")
+    print(f"Hidden Size: {spec.hidden_size}")
+    print(f"Num Layers: {len(spec.layers)}")
+    if hasattr(cfg, "num_attention_heads"):
+        print(f"Num Attention Heads: {cfg.num_attention_heads}")
+        print(f"Num KV Heads: {cfg.num_key_value_heads}")
+        print(f"Head Dimension: {cfg.head_dim}")
+    else:      # layers of several kinds: say which
+        kinds = [layer.mixer.kind for layer in spec.layers]
+        print("Mixers: " + ", ".join(f"{kinds.count(kind)} x {kind}" for kind in dict.fromkeys(kinds)))
     seed = args.seed if args.seed is not None else time.time_ns() & 0xFFFFFFFF
     session = model.new_session(capacity=args.context_capacity, seed=seed)
     print(f"Model initialized on {model.device}; context capacity: {session.capacity} tokens.\n")

@@ -1,0 +1,274 @@
+"""The Tirurax decoder in the engine against the plain implementation (`plain_tirurax`), in
+float32 and bfloat16: whole prompts, prompts then tokens one by one, portions down to two
+tokens, batches of unequal requests with slots and pages used again, long decoding over
+chunk edges and page borders, the first tokens of a sequence, a token far back, greedy
+generation through the entry point, and the framework's own random-weights folder."""
+import json
+
+import pytest
+import torch
+
+import plain_tirurax as plain
+from helpers import assert_close_bf16, assert_close_f32
+from tirurax_helpers import CONFIGS, ids, sharp_weights, write_folder
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+NAMES = ["A", "B"]
+LENGTHS = {"A": [150, 1, 49, 75], "B": [210, 2, 101, 64]}
+# bfloat16 engine against the float64 oracle on these order-one weights: root-mean-square
+# error relative to the logits' root-mean-square, and largest error relative to the
+# largest logit (a recurrent state and several renormalised sublayers round more often
+# than the layers of the other architecture's tests, and the largest error is taken over
+# up to 300 x 211 logits; the largest seen are 1.9 % and 5.2 %)
+BF16_RMS, BF16_MAX = 4e-2, 8e-2
+
+
+def close(dtype, actual, expected, what):
+    if dtype == "float32":
+        return assert_close_f32(actual, expected, what)
+    return assert_close_bf16(actual, expected, what, rms_rel=BF16_RMS, max_rel=BF16_MAX)
+
+
+@pytest.fixture(scope="module")
+def weights():
+    return {name: sharp_weights(CONFIGS[name], seed=20 + i) for i, name in enumerate(NAMES)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory, weights):
+    root = tmp_path_factory.mktemp("tirurax")
+    return {name: write_folder(root / name, CONFIGS[name], weights[name]) for name in NAMES}
+
+
+@pytest.fixture(scope="module")
+def models(folders):
+    import edge_infer_amd as ei
+    cache = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in cache:
+            cache[(name, dtype)] = ei.load_model(folders[name], dtype=dtype)
+        return cache[(name, dtype)]
+    return get
+
+
+def requests_for(name, seed=5):
+    return [ids(CONFIGS[name]["vocab"], n, seed + i) for i, n in enumerate(LENGTHS[name])]
+
+
+@pytest.fixture(scope="module")
+def references(weights):
+    return {name: [plain.forward(CONFIGS[name], weights[name], r) for r in requests_for(name)]
+            for name in NAMES}
+
+
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_whole_prompts(models, references, name, dtype):
+    import edge_infer_amd as ei
+    session = ei.Session(models(name, dtype), max_tokens=512)
+    for request, ref in zip(requests_for(name), references[name]):
+        slot = session.begin()
+        logits = session.step([(slot, request, list(range(len(request))))])
+        close(dtype, logits, ref, f"{name} {dtype} whole {len(request)}")
+        session.end(slot)
+    session.cache.check()
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_prompt_then_tokens_one_by_one(models, references, name, dtype, graphs):
+    """The decoded tokens pass chunk edges (24, 100, 7) and a page border (64, 128)."""
+    import edge_infer_amd as ei
+    session = ei.Session(models(name, dtype), max_tokens=512, graphs=graphs)
+    for request, ref in zip(requests_for(name), references[name]):
+        cut = max(1, len(request) - 60)
+        slot = session.begin()
+        rows = [session.step([(slot, request[:cut], [cut - 1])])]
+        rows += [session.step([(slot, [token], [0])]) for token in request[cut:]]
+        close(dtype, torch.cat(rows), ref[cut - 1:], f"{name} {dtype} tail of {len(request)}")
+        session.end(slot)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("sizes", [(2, 2, 3, 2), (1, 5, 64, 2, 7), (63, 2, 65), (24, 100, 7)])
+def test_portions(models, references, name, dtype, sizes):
+    """A prompt cut into portions (the given sizes in turn, down to two tokens and one): every
+    position's logits are those of the whole prompt."""
+    import edge_infer_amd as ei
+    session = ei.Session(models(name, dtype), max_tokens=512)
+    request, ref = requests_for(name)[0], references[name][0]
+    slot = session.begin()
+    rows, at, turn = [], 0, 0
+    while at < len(request):
+        take = min(sizes[turn % len(sizes)], len(request) - at)
+        rows.append(session.step([(slot, request[at:at + take], list(range(take)))]))
+        at, turn = at + take, turn + 1
+    close(dtype, torch.cat(rows), ref, f"{name} {dtype} portions {sizes}")
+    session.end(slot)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_batches_of_unequal_requests_with_slots_and_pages_used_again(models, references, name, dtype):
+    """Requests of unequal lengths start together and are decoded together; the shorter end
+    earlier and their slots and pages go back; a second and a third batch then run in what was
+    freed (the cache has room for little more than one batch)."""
+    import edge_infer_amd as ei
+    requests, refs = requests_for(name), references[name]
+    tail = 20
+    session = ei.Session(models(name, dtype), max_tokens=64 * 9, max_seqs=4)
+    for batch in ([0, 1, 2, 3], [3, 2, 0], [1, 0, 3, 2]):
+        slots = {i: session.begin() for i in batch}
+        cuts = {i: max(1, len(requests[i]) - tail) for i in batch}
+        got = {i: [] for i in batch}
+        logits = session.step([(slots[i], requests[i][:cuts[i]], [cuts[i] - 1]) for i in batch])
+        for row, i in enumerate(batch):
+            got[i].append(logits[row:row + 1])
+        at = dict(cuts)
+        live = [i for i in batch if at[i] < len(requests[i])]
+        for i in batch:
+            if i not in live:
+                session.end(slots[i])
+        while live:
+            logits = session.step([(slots[i], [requests[i][at[i]]], [0]) for i in live])
+            for row, i in enumerate(live):
+                got[i].append(logits[row:row + 1])
+                at[i] += 1
+            for i in [i for i in live if at[i] == len(requests[i])]:
+                session.end(slots[i])
+                live.remove(i)
+        for i in batch:
+            close(dtype, torch.cat(got[i]), refs[i][cuts[i] - 1:],
+                  f"{name} {dtype} request {i} in batch {batch}")
+        session.cache.check()
+    assert session.cache.slots.n_free == 4
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_long_decoding_from_the_first_token(models, weights, name, dtype):
+    """One token, then 299 more one by one, from graphs: every chunk edge and four page
+    borders are passed while decoding, and the state is carried 300 times."""
+    import edge_infer_amd as ei
+    request = ids(CONFIGS[name]["vocab"], 300, 77)
+    ref = plain.forward(CONFIGS[name], weights[name], request)
+    session = ei.Session(models(name, dtype), max_tokens=320)
+    slot = session.begin()
+    rows = [session.step([(slot, [token], [0])]) for token in request]
+    close(dtype, torch.cat(rows), ref, f"{name} {dtype} 300 tokens one by one")
+    if session.graphs:     # (B in bfloat16 has a product of width 12, which the library multiplies)
+        assert session.graph_replays > 250
+    else:
+        assert (name, dtype) == ("B", "bfloat16")
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_a_token_far_back_shows(tmp_path, name):
+    """Delta layers that forget slowly: two prompts that differ in their third token alone
+    still differ at position 400, by far more than the tolerance, and the engine follows the
+    oracle for both, whole, in portions and decoded."""
+    import edge_infer_amd as ei
+    cfg = CONFIGS[name]
+    tensors = sharp_weights(cfg, seed=31, slow_decay=True)
+    model = ei.load_model(write_folder(tmp_path / "slow", cfg, tensors), dtype="float32")
+    base = ids(cfg["vocab"], 401, 3)
+    other = list(base)
+    other[2] = (base[2] + 1) % cfg["vocab"]
+    refs = [plain.forward(cfg, tensors, r)[-1:] for r in (base, other)]
+    gap = (refs[0] - refs[1]).abs().max().item() / refs[0].abs().max().item()
+    assert gap > 1e-3, f"the test's weights do not carry the third token to the end ({gap:.1e})"
+    session = ei.Session(model, max_tokens=1024)
+    for request, ref in zip((base, other), refs):
+        slot = session.begin()
+        close("float32", session.step([(slot, request, [400])]), ref, "far token, whole")
+        session.end(slot)
+        slot = session.begin()
+        session.step([(slot, request[:130], [])])
+        session.step([(slot, request[130:390], [])])
+        for token in request[390:400]:
+            session.step([(slot, [token], [])])
+        close("float32", session.step([(slot, request[400:], [0])]), ref, "far token, decoded")
+        session.end(slot)
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_greedy_generation_through_the_entry_point(models, weights, name):
+    """`Session.generate_batch` (the scheduler, sampler and step function together) gives the
+    oracle's greedy tokens in float32."""
+    import edge_infer_amd as ei
+    cfg = CONFIGS[name]
+    prompts = [ids(cfg["vocab"], n, 40 + n) for n in (5, 1, 30)]
+    session = ei.Session(models(name, "float32"), max_tokens=512, max_seqs=3)
+    got = session.generate_batch(prompts, max_new_tokens=12, temperature=0.0)
+    for prompt, tokens in zip(prompts, got):
+        sequence = list(prompt)
+        for token in tokens:
+            logits = plain.forward(cfg, weights[name], sequence)[-1]
+            best = logits.argmax().item()
+            if token != best:       # only a tie within float32's reach may differ
+                assert (logits[best] - logits[token]).item() <= 2e-5 * logits.abs().max().item()
+            sequence.append(token)
+        assert len(tokens) == 12
+
+
+def test_model_type_through_the_python_entry(folders, weights):
+    from edge_infer_amd.api import Model
+    model = Model.from_pretrained(folders["A"], "tirurax_fp32")
+    session = model.new_session(capacity=128, max_batch=2)
+    prompt = ids(CONFIGS["A"]["vocab"], 9, 1)
+    tokens = session.generate(prompt, None, max_length=len(prompt) + 4, temperature=0.0)
+    logits = plain.forward(CONFIGS["A"], weights["A"], prompt)[-1]
+    assert tokens[0] == logits.argmax().item() and len(tokens) == 4
+
+
+def test_random_weights_folder_of_the_framework(tmp_path):
+    """`write_model_folder` writes a Tirurax folder that reads back to the same configuration
+    and runs; its tensors carry the checkpoint's names."""
+    import edge_infer_amd as ei
+    from safetensors.torch import load_file
+    from tirurax_helpers import tensor_shapes
+    cfg = ei.config.TiruraxConfig.from_dict(CONFIGS["B"])
+    folder = ei.write_model_folder(tmp_path / "random", cfg, seed=2)
+    assert ei.read_config(folder)[1] == cfg
+    tensors = load_file(str(folder / "model.safetensors"))
+    assert {k: tuple(v.shape) for k, v in tensors.items()} == \
+        {k: shape for k, (shape, _) in tensor_shapes(CONFIGS["B"]).items()}
+    model = ei.load_model(folder, dtype="bfloat16")
+    session = ei.Session(model, max_tokens=128)
+    slot = session.begin()
+    request = ids(CONFIGS["B"]["vocab"], 70, 9)
+    logits = session.step([(slot, request, [69])])
+    ref = plain.forward(json.loads((folder / "config.json").read_text()), tensors, request)[-1:]
+    close("bfloat16", logits, ref, "random folder")
+
+
+def test_the_replay_program_runs_a_tirurax_folder(folders, weights, tmp_path):
+    """`bin/trace_run` chooses the model class by config.json and writes the step's logits."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    import numpy as np
+    root = Path(__file__).resolve().parents[1]
+    request = ids(CONFIGS["A"]["vocab"], 30, 8)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": request[:28], "want": [0, 27]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": request[28:29], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": request[29:], "want": [0]}], "end": ["x"]}]
+    done = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model",
+                           str(folders["A"]), "--dtype", "float32", "--out", str(tmp_path),
+                           "--max-tokens", "64"], input="\n".join(json.dumps(s) for s in steps),
+                          capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert [l for l in done.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert not (tmp_path / "1.f32").exists()
+    ref = plain.forward(CONFIGS["A"], weights["A"], request)
+    vocab = CONFIGS["A"]["vocab"]
+    first = torch.from_numpy(np.fromfile(tmp_path / "0.f32", dtype="<f4").reshape(2, vocab))
+    last = torch.from_numpy(np.fromfile(tmp_path / "2.f32", dtype="<f4").reshape(1, vocab))
+    assert_close_f32(first, ref[[0, 27]], "replayed prompt")
+    assert_close_f32(last, ref[29:], "replayed token")
