@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
                     [--shape 8b|0.6b|32b] [--only decode|prefill|generate] [--prompt P]
-                    [--with-32b] [--peaks]
+                    [--with-32b] [--peaks] [--design tirurax [--design-shape 1k|2k|4k]]
 
 Prints one JSON line.  `value` is decoded tokens per second at the given batch after
 512-token prompts (one step = one decode step of the whole batch: the model, greedy
@@ -20,6 +20,11 @@ stand `<name>_ms` (a step), `<name>_GB` (what the step has to read, or `_TFLOP`:
 to multiply), `<name>_frac` (of the published peak) and `<name>_frac_measured` (of what the
 chip at hand gives).  `decode_b8_launches` and `decode_b8_launch_floor_ms`: the kernel launches
 of a decode step, and what a graph of as many launches of a kernel that does nothing takes.
+`--design tirurax` measures another workload and leaves the default one as it is: prefill
+(one prompt of 2,048 tokens, and 8 of 512) and decode (batch 1, 8 and 64 after 512-token
+prompts) of a Tirurax model of real layer sizes (gated-delta and chunked-attention layers in
+turn, dense feed-forward of four widths) beside a Qwen3 model of the same width, layers,
+heads and parameter count, as one JSON line.
 Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
 ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s; `measured_peaks` (and `--peaks` alone) say what
 a plain read kernel and a loop of matrix-core products reach on the GPU at hand, and the
@@ -323,6 +328,96 @@ def other_shape_points(args, itemsize, peaks):
     return points
 
 
+# name: (layers, width, delta value heads, delta key heads, attention heads, attention kv heads,
+#        head size, attention chunk, vocabulary)
+DESIGN_SHAPES = {
+    "1k": (8, 1024, 16, 8, 16, 8, 64, 512, 32000),
+    "2k": (8, 2048, 16, 8, 16, 4, 128, 1024, 32000),
+    "4k": (4, 4096, 32, 16, 32, 8, 128, 1024, 32000),
+}
+
+
+def design_configs(shape):
+    """(Tirurax configuration, Qwen3 configuration) of equal width, layers, heads, head size
+    and feed-forward parameters (a gated feed-forward of 2/3 the dense one's width has as many)."""
+    import edge_infer_amd as ei
+    from edge_infer_amd.config import TiruraxConfig
+    layers, width, d_heads, d_kv, a_heads, a_kv, dim, chunk, vocab = DESIGN_SHAPES[shape]
+    ff = 4 * width
+    delta = {"type": "delta", "mixer": {"heads": d_heads, "kv_heads": d_kv, "dim": dim,
+                                        "vdim": dim, "conv": 4},
+             "mlp": {"kind": "dense", "ff": ff}}
+    attention = {"type": "attention", "mixer": {"heads": a_heads, "kv_heads": a_kv, "dim": dim,
+                                                "vdim": dim, "scale": dim ** -0.5,
+                                                "mask": {"size": chunk}},
+                 "mlp": {"kind": "dense", "ff": ff}}
+    new = TiruraxConfig.from_dict({"architecture": "Tirurax", "vocab": vocab, "width": width,
+                                   "norm": {"eps": 1e-6},
+                                   "layers": [delta if i % 2 == 0 else attention
+                                              for i in range(layers)]})
+    old = ei.Qwen3Config(vocab_size=vocab, hidden_size=width, num_hidden_layers=layers,
+                         num_attention_heads=a_heads, num_key_value_heads=a_kv, head_dim=dim,
+                         intermediate_size=(2 * ff // 3 + 255) // 256 * 256,
+                         max_position_embeddings=40960, bos_token_id=0, eos_token_id=1,
+                         rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False)
+    return new, old
+
+
+def measure_prompts(model, vocab, batch, tokens, repeats=3):
+    """Best ms of one step over `batch` prompts of `tokens` tokens that start together."""
+    import types
+    import torch
+    import edge_infer_amd as ei
+    session = ei.Session(model, max_tokens=batch * tokens, max_seqs=batch)
+    prompts = synthetic_prompts(types.SimpleNamespace(vocab_size=vocab), batch, tokens, seed=11)
+    best = None
+    for _ in range(repeats + 1):
+        slots = [session.begin() for _ in range(batch)]
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        session.step([(s, p, [tokens - 1]) for s, p in zip(slots, prompts)], copy=False)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        for s in slots:
+            session.end(s)
+        best = elapsed if best is None else min(best, elapsed)
+    del session
+    torch.cuda.empty_cache()
+    return 1000.0 * best
+
+
+def design_comparison(args):
+    """Prefill and decode of the Tirurax shape and of the Qwen3 model of equal size."""
+    import types
+    import torch
+    import edge_infer_amd as ei
+    new, old = design_configs(args.design_shape)
+    vocab = new.vocab
+    sizes = types.SimpleNamespace(vocab_size=vocab)
+    record = {"only": "design", "design": "tirurax", "shape": args.design_shape,
+              "dtype": args.dtype, "layers": len(new.layers), "width": new.width}
+    which = {"tirurax": new, "qwen3": old}
+    if args.design_only:
+        which = {args.design_only: which[args.design_only]}
+    for name, cfg in which.items():
+        model = ei.random_model(cfg, seed=2, dtype=args.dtype)
+        torch.cuda.synchronize()
+        out = {"weight_GB": round(model.weight_bytes() / 1e9, 3)}
+        for batch, tokens in ((1, 2048), (8, 512)):
+            ms = measure_prompts(model, vocab, batch, tokens)
+            out[f"prefill_{batch}x{tokens}_ms"] = round(ms, 3)
+            out[f"prefill_{batch}x{tokens}_tokens_per_s"] = round(batch * tokens * 1000.0 / ms, 1)
+        for batch in (1, 8, 64):
+            ms, _, median = measure_decode(model, sizes, batch, args.steps, args.warmup)
+            out[f"decode_b{batch}_ms"] = round(ms, 4)
+            out[f"decode_b{batch}_tokens_per_s"] = round(batch * 1000.0 / ms, 1)
+        record[name] = out
+        del model
+        torch.cuda.empty_cache()
+    print(json.dumps(record))
+    return 0
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -351,6 +446,12 @@ def main():
                         help="leave the 32B shape (decode at batch 1 and 16, prefill) out of `points`")
     parser.add_argument("--peaks", action="store_true",
                         help="measure the read and matrix-core yardsticks only")
+    parser.add_argument("--design", choices=["tirurax"], default=None,
+                        help="measure this design beside the Qwen3 model of equal size instead "
+                             "of the default workload")
+    parser.add_argument("--design-shape", choices=sorted(DESIGN_SHAPES), default="2k")
+    parser.add_argument("--design-only", choices=["tirurax", "qwen3"], default=None,
+                        help="with --design: one of the two models only (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -362,6 +463,8 @@ def main():
         print(json.dumps({"only": "peaks", **measure_peaks(),
                           "published": {"hbm_GBs": HBM_PEAK_GBS, "mfma_bf16_TFLOPs": PEAK_TFLOPS["bfloat16"]}}))
         return 0
+    if args.design:
+        return design_comparison(args)
     cfg = model_config(args.shape, args.layers)
     full_layers = SHAPES[args.shape][0]
     model = ei.random_model(cfg, seed=2, dtype=args.dtype)

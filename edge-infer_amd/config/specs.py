@@ -78,13 +78,6 @@ class AttentionSpec:
     def out_width(self) -> int:
         return self.n_heads * self.v_dim
 
-    @property
-    def extended(self) -> bool:
-        """Whether the mixer uses anything beyond rotary/windowed attention with per-head
-        norms and equal widths (what the matrix-core kernels take)."""
-        return (self.v_dim != self.head_dim or self.qk_norm_scope != "head"
-                or self.chunk is not None or self.distance_slope_range is not None or self.sink)
-
 
 @dataclass(frozen=True)
 class GatedMLPSpec:

@@ -25,6 +25,16 @@ namespace {
 constexpr int kTile = 16;          // keys per MFMA tile
 constexpr float kLowest = -1.0e30f;
 
+// Options beyond causal, windowed attention (the EXT instantiations of the kernels; the plain
+// ones are compiled without any of this): `chunk` > 0: a query at p sees key t only if
+// t / chunk == p / chunk; `slopes` (per query head, or null): slope * (p - t) is taken off the
+// scaled score; `sinks` (per query head, or null): exp(sink) joins the softmax's denominator.
+struct AttnExtra {
+  int chunk;
+  const float* slopes;
+  const float* sinks;
+};
+
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
@@ -55,7 +65,7 @@ struct DecodePrep {
 // PREP: q is not read; the block forms its queries and the position's key and value itself
 // (the block of slice 0 and head block 0 stores them; the wave that meets the position in
 // its tile takes them from LDS, since the store of another block may not have landed).
-template <int D, int GB, int W, bool PREP>
+template <int D, int GB, int W, bool PREP, bool EXT>
 __global__ void __launch_bounds__(W * EI_WAVE)
 attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                    const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ row_pos,
@@ -63,7 +73,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
                    int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o,
                    float* __restrict__ part_ml, int nq, int nkv, int head_blocks, int window,
                    float scale, int n_splits, const int32_t* __restrict__ longest,
-                   DecodePrep prep) {
+                   DecodePrep prep, AttnExtra extra) {
   constexpr int DJ = D / 32;            // MFMA steps over the head dimension
   constexpr int LPR = D / 8;            // lanes that cover one value row with 16-byte loads
   constexpr int KPI = EI_WAVE / LPR;    // value rows per load instruction
@@ -184,7 +194,10 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
     q_reg[j] = *reinterpret_cast<bf16x8*>(&z);
   }
 
-  const int lo_key = window > 0 ? max(0, pos - window + 1) : 0;
+  int lo_key_of = window > 0 ? max(0, pos - window + 1) : 0;
+  if constexpr (EXT)
+    if (extra.chunk > 0) lo_key_of = max(lo_key_of, pos / extra.chunk * extra.chunk);
+  const int lo_key = lo_key_of;
   const int first_tile = lo_key / kTile, last_tile = pos / kTile;
   const int total_tiles = last_tile - first_tile + 1;
   // slices are cut at page boundaries so that they do not depend on the tile size
@@ -196,7 +209,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   // the later slices of a short sequence are empty.  Without it (or with a window, where the
   // ranges start at different pages) every sequence is cut into n_splits equal parts.
   int per = (pages + n_splits - 1) / n_splits;
-  if (longest != nullptr && window <= 0) {
+  if (longest != nullptr && window <= 0 && !(EXT && extra.chunk > 0)) {
     const int most_pages = (*longest + EI_PAGE - 1) / EI_PAGE;
     per = max(1, (most_pages + n_splits - 1) / n_splits);
   }
@@ -208,6 +221,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   (void)total_tiles;
 
   float m_run = kLowest, l_run = 0.f;              // state of head r16 (same in all four c)
+  float slope = 0.f;                               // of head r16
+  if constexpr (EXT)
+    if (extra.slopes && r16 < heads_here) slope = extra.slopes[head0 + r16];
   float acc[GB][8];
 #pragma unroll
   for (int h = 0; h < GB; ++h)
@@ -265,7 +281,10 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
     for (int r = 0; r < 4; ++r) {
       const int key = key0 + 4 * c + r;
       const bool visible = key <= pos && key >= lo_key;
-      sc[r] = visible ? s[r] * scale : -INFINITY;
+      if constexpr (EXT)
+        sc[r] = visible ? fmaf(-slope, static_cast<float>(pos - key), s[r] * scale) : -INFINITY;
+      else
+        sc[r] = visible ? s[r] * scale : -INFINITY;
       tile_max = fmaxf(tile_max, sc[r]);
     }
     tile_max = ei::rows_max(tile_max);
@@ -353,6 +372,15 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
       o += o_lds[w][h][d] * f;
     }
     const int head = head0 + h;
+    if constexpr (EXT) {
+      if (extra.sinks && split == 0) {     // one more term of the denominator, once a row
+        const float sink = extra.sinks[head];
+        const float m_all = fmaxf(m, sink), f = expf(m - m_all);
+        l = l * f + expf(sink - m_all);
+        o *= f;
+        m = m_all;
+      }
+    }
     if (n_splits == 1) {
       out[(static_cast<size_t>(row) * nq + head) * D + d] =
           ei::from_f32<bf16_t>(l > 0.f ? o / l : 0.f);
@@ -436,7 +464,7 @@ constexpr int kPageBuffers = 3;
 // a lane and a trip through LDS) was a quarter of a page's vector work.
 constexpr float kLazyRise = 8.f;
 
-template <int D, int HB, int KW>
+template <int D, int HB, int KW, bool EXT>
 __global__ void __launch_bounds__(kPrefillThreads, 2)
 attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                          const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ item_seq,
@@ -445,7 +473,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
                          const int32_t* __restrict__ row_pos,
                          const int32_t* __restrict__ page_table, int table_width,
                          bf16_t* __restrict__ out, int nq, int nkv, int window, float scale,
-                         int pair) {
+                         int pair, AttnExtra extra) {
   constexpr int SJ = D / 16;             // 16-wide steps over d for the scores
   constexpr int DB = D / 32;             // 32-wide output blocks over d
   constexpr int CHUNKS = D / 8;          // 16-byte chunks of a row
@@ -557,7 +585,20 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   }
 
   const int first_pos = row_pos[row0], last_pos = row_pos[row0 + npos - 1];
-  const int lo_key = window > 0 ? max(0, first_pos - window + 1) : 0;
+  int lo_key_of = window > 0 ? max(0, first_pos - window + 1) : 0;
+  const int chunk = EXT ? extra.chunk : 0;
+  // (EXT) the first key of this lane's row's own chunk, and the slope of the wave's head in
+  // units of the raw score (the scale is positive)
+  int chunk_lo = 0;
+  float slope_raw = 0.f;
+  if constexpr (EXT) {
+    if (chunk > 0) {
+      lo_key_of = max(lo_key_of, first_pos / chunk * chunk);
+      chunk_lo = pos_q >= 0 ? pos_q / chunk * chunk : 0;
+    }
+    if (extra.slopes) slope_raw = extra.slopes[head] / scale;
+  }
+  const int lo_key = lo_key_of;
   const int lo_page = lo_key / EI_PAGE, hi_page = last_pos / EI_PAGE;
   const bool wave_rows_valid = pw * kWideRows + kWideRows <= npos;
   const int wave_min_pos = wave_rows_valid ? row_pos[row0 + pw * kWideRows] : -1;
@@ -651,6 +692,19 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
+    if constexpr (EXT) {
+      if (slope_raw != 0.f) {
+#pragma unroll
+        for (int kb = 0; kb < KBL; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int key = key_base + (kw * KBL + kb) * 32 + 8 * i + 4 * half + r;
+              s[kb][4 * i + r] = fmaf(-slope_raw, static_cast<float>(pos_q - key), s[kb][4 * i + r]);
+            }
+      }
+    }
     if (MASKED) {
       // (an empty statement the compiler may not move: it keeps this a branch, which all but
       // the last pages of a causal prompt jump over, instead of 128 predicated instructions)
@@ -662,7 +716,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int key = key_base + (kw * KBL + kb) * 32 + 8 * i + 4 * half + r;
-            const bool visible = key <= pos_q && (window <= 0 || key > pos_q - window);
+            bool visible = key <= pos_q && (window <= 0 || key > pos_q - window);
+            if constexpr (EXT) visible = visible && key >= chunk_lo;
             if (!visible) s[kb][4 * i + r] = -INFINITY;     // (pos_q = -1: a row that is not there)
           }
     }
@@ -745,14 +800,19 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   // (the wave's keys of a page: KBL blocks of 32 from block kw * KBL on)
   auto page_seen = [&](const int page) __attribute__((always_inline)) {
     const int key_lo = page * EI_PAGE + kw * KBL * 32, key_hi = key_lo + KBL * 32 - 1;
-    return wave_has_rows && key_lo <= wave_last_pos &&
-           (window <= 0 || !wave_rows_valid || key_hi > wave_min_pos - window);
+    bool seen = wave_has_rows && key_lo <= wave_last_pos &&
+                (window <= 0 || !wave_rows_valid || key_hi > wave_min_pos - window);
+    if constexpr (EXT)     // wholly before the chunk of the wave's first row: no row sees it
+      if (chunk > 0 && wave_rows_valid) seen = seen && key_hi >= wave_min_pos / chunk * chunk;
+    return seen;
   };
   auto scores_of = [&](const int page, const int buf) __attribute__((always_inline)) {
     const int key_base = page * EI_PAGE;
     const int key_lo = key_base + kw * KBL * 32, key_hi = key_lo + KBL * 32 - 1;
-    const bool no_mask = wave_rows_valid && key_hi <= wave_min_pos &&
-                         (window <= 0 || key_lo > wave_max_pos - window);
+    bool no_mask = wave_rows_valid && key_hi <= wave_min_pos &&
+                   (window <= 0 || key_lo > wave_max_pos - window);
+    if constexpr (EXT)     // every key lies in the chunk of the wave's last row, so of all rows
+      if (chunk > 0) no_mask = no_mask && key_lo >= wave_max_pos / chunk * chunk;
     scores(key_base, buf, !no_mask);
   };
   using Both = std::integral_constant<int, LOADS>;
@@ -784,7 +844,17 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
                                                          __float_as_uint(l_run), false, false);
     l_wave = __uint_as_float(both.x) + __uint_as_float(both.y);
   }
-  float own_factor = l_wave > 0.f ? 1.f / l_wave : 0.f;   // what this wave's output is scaled by
+  float sink_fold = 1.f;       // (EXT) what taking the sink in rescales this wave's output by
+  if constexpr (EXT) {
+    if (extra.sinks && kw == 0) {          // one more term of the denominator, once a row
+      const float sink_l2 = extra.sinks[head] * 1.4426950408889634f;
+      const float m_new = fmaxf(m_run, sink_l2);
+      sink_fold = __builtin_amdgcn_exp2f(m_run - m_new);
+      l_wave = l_wave * sink_fold + __builtin_amdgcn_exp2f(sink_l2 - m_new);
+      m_run = m_new;
+    }
+  }
+  float own_factor = l_wave > 0.f ? sink_fold / l_wave : 0.f;   // what this wave's output is scaled by
   float other_factor = 0.f;                               // and the handed-over one
   if constexpr (KW == 2) {
     // The wave of the second half of every page's keys hands its state to the wave of the
@@ -811,7 +881,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
       const float f_other = __builtin_amdgcn_exp2f(m_other - m);
       const float l = l_wave * f_own + l_other * f_other;
       const float inv = l > 0.f ? 1.f / l : 0.f;
-      own_factor = f_own * inv;
+      own_factor = sink_fold * f_own * inv;
       other_factor = f_other * inv;
     }
   }
@@ -900,31 +970,32 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o,
   }
 }
 
-template <int D, int GB, bool PREP>
+template <int D, int GB, bool PREP, bool EXT>
 void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k,
                    const bf16_t* v, const int32_t* row_pos, const int32_t* row_seq,
                    const int32_t* page_table, int table_width, bf16_t* out, float* part_o,
                    float* part_ml, int nq, int nkv, int head_blocks, int window, float scale,
-                   int n_splits, int waves, const int32_t* longest, const DecodePrep& prep) {
+                   int n_splits, int waves, const int32_t* longest, const DecodePrep& prep,
+                   const AttnExtra& extra) {
   if constexpr (GB <= 4) {               // the caller gives 16 waves at most 4 heads a block
     if (waves == 16) {
-      attn_decode_kernel<D, GB, 16, PREP><<<grid, 16 * EI_WAVE, 0, stream>>>(
+      attn_decode_kernel<D, GB, 16, PREP, EXT><<<grid, 16 * EI_WAVE, 0, stream>>>(
           q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
-          head_blocks, window, scale, n_splits, longest, prep);
+          head_blocks, window, scale, n_splits, longest, prep, extra);
       return;
     }
   }
   if constexpr (GB <= 8) {               // and 8 waves at most 8
     if (waves == 8) {
-      attn_decode_kernel<D, GB, 8, PREP><<<grid, 8 * EI_WAVE, 0, stream>>>(
+      attn_decode_kernel<D, GB, 8, PREP, EXT><<<grid, 8 * EI_WAVE, 0, stream>>>(
           q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
-          head_blocks, window, scale, n_splits, longest, prep);
+          head_blocks, window, scale, n_splits, longest, prep, extra);
       return;
     }
   }
-  attn_decode_kernel<D, GB, 4, PREP><<<grid, 4 * EI_WAVE, 0, stream>>>(
+  attn_decode_kernel<D, GB, 4, PREP, EXT><<<grid, 4 * EI_WAVE, 0, stream>>>(
         q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
-        head_blocks, window, scale, n_splits, longest, prep);
+        head_blocks, window, scale, n_splits, longest, prep, extra);
 }
 
 }  // namespace
@@ -937,16 +1008,16 @@ extern "C" int ei_attn_prefill_mfma_positions(int G) {
   return kWideRows * (kPrefillWaves / HB);
 }
 
-template <int D, int HB, int KW>
+template <int D, int HB, int KW, bool EXT>
 static void launch_prefill(int blocks, hipStream_t stream, const bf16_t* q, const bf16_t* k,
                                 const bf16_t* v, const int32_t* item_seq,
                                 const int32_t* item_row0, const int32_t* item_npos, int n_items,
                                 const int32_t* row_pos, const int32_t* page_table,
                                 int table_width, bf16_t* out, int nq, int nkv, int window,
-                                float scale, int pair) {
-  attn_prefill_kernel<D, HB, KW><<<blocks, kPrefillThreads, 0, stream>>>(
+                                float scale, int pair, const AttnExtra& extra) {
+  attn_prefill_kernel<D, HB, KW, EXT><<<blocks, kPrefillThreads, 0, stream>>>(
       q, k, v, item_seq, item_row0, item_npos, n_items, row_pos, page_table, table_width, out,
-      nq, nkv, window, scale, pair);
+      nq, nkv, window, scale, pair, extra);
 }
 
 // q, out: [N, nq, D] bfloat16; items: (sequence, first packed row, positions), each holding
@@ -955,13 +1026,12 @@ static void launch_prefill(int blocks, hipStream_t stream, const bf16_t* q, cons
 // caller, who makes them, is bound to it).  pair_items: a block may take item i and item
 // n_items - 1 - i one after the other, which pays where those sums are about equal (the
 // items of one prompt, longest first) and enough blocks remain.
-extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, const void* v_pages,
-                                         const int32_t* item_seq, const int32_t* item_row0,
-                                         const int32_t* item_npos, int n_items,
-                                         const int32_t* row_pos, const int32_t* page_table,
-                                         int table_width, void* out, int nq, int nkv, int D,
-                                         int window, float scale, int key_ways, int pair_items,
-                                         hipStream_t stream) {
+static int prefill_launch(const void* q, const void* k_pages, const void* v_pages,
+                          const int32_t* item_seq, const int32_t* item_row0,
+                          const int32_t* item_npos, int n_items, const int32_t* row_pos,
+                          const int32_t* page_table, int table_width, void* out, int nq, int nkv,
+                          int D, int window, float scale, int key_ways, int pair_items,
+                          const AttnExtra* extra, hipStream_t stream) {
   EI_REQUIRE(n_items > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes");
   EI_REQUIRE(D == 64 || D == 128, "attention_prefill: this kernel takes head_dim 64 or 128");
   EI_REQUIRE(q && k_pages && v_pages && item_seq && item_row0 && item_npos && row_pos &&
@@ -992,16 +1062,22 @@ extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, con
   const bf16_t* kk = static_cast<const bf16_t*>(k_pages);
   const bf16_t* vv = static_cast<const bf16_t*>(v_pages);
   bf16_t* oo = static_cast<bf16_t*>(out);
+  const AttnExtra none{0, nullptr, nullptr};
+#define EI_PREFILL_KW(DD, HH, KK)                                                             \
+  do {                                                                                        \
+    if (extra)                                                                                \
+      launch_prefill<DD, HH, KK, true>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq, \
+                                       item_row0, item_npos, n_items, row_pos, page_table,    \
+                                       table_width, oo, nq, nkv, window, scale, pair, *extra); \
+    else                                                                                      \
+      launch_prefill<DD, HH, KK, false>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq, \
+                                        item_row0, item_npos, n_items, row_pos, page_table,   \
+                                        table_width, oo, nq, nkv, window, scale, pair, none); \
+  } while (0)
 #define EI_PREFILL(DD, HH)                                                                    \
   do {                                                                                        \
-    if (key_ways == 2)                                                                        \
-      launch_prefill<DD, HH, 2>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq,       \
-                                item_row0, item_npos, n_items, row_pos, page_table,           \
-                                table_width, oo, nq, nkv, window, scale, pair);               \
-    else                                                                                      \
-      launch_prefill<DD, HH, 1>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq,       \
-                                item_row0, item_npos, n_items, row_pos, page_table,           \
-                                table_width, oo, nq, nkv, window, scale, pair);               \
+    if (key_ways == 2) EI_PREFILL_KW(DD, HH, 2);                                              \
+    else EI_PREFILL_KW(DD, HH, 1);                                                            \
   } while (0)
   if (D == 64) {
     if (HB == 4) EI_PREFILL(64, 4); else if (HB == 2) EI_PREFILL(64, 2); else EI_PREFILL(64, 1);
@@ -1009,7 +1085,36 @@ extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, con
     if (HB == 4) EI_PREFILL(128, 4); else if (HB == 2) EI_PREFILL(128, 2); else EI_PREFILL(128, 1);
   }
 #undef EI_PREFILL
+#undef EI_PREFILL_KW
   EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, const void* v_pages,
+                                         const int32_t* item_seq, const int32_t* item_row0,
+                                         const int32_t* item_npos, int n_items,
+                                         const int32_t* row_pos, const int32_t* page_table,
+                                         int table_width, void* out, int nq, int nkv, int D,
+                                         int window, float scale, int key_ways, int pair_items,
+                                         hipStream_t stream) {
+  return prefill_launch(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
+                        page_table, table_width, out, nq, nkv, D, window, scale, key_ways,
+                        pair_items, nullptr, stream);
+}
+
+// The same with the options of `AttnExtra`: chunk (0: none), slopes and sinks (float32 [nq] on
+// the device, or null).
+extern "C" int ei_attention_prefill_mfma_ext(
+    const void* q, const void* k_pages, const void* v_pages, const int32_t* item_seq,
+    const int32_t* item_row0, const int32_t* item_npos, int n_items, const int32_t* row_pos,
+    const int32_t* page_table, int table_width, void* out, int nq, int nkv, int D, int window,
+    float scale, int key_ways, int pair_items, int chunk, const float* slopes,
+    const float* sinks, hipStream_t stream) {
+  EI_REQUIRE(chunk >= 0, "attention_prefill: negative chunk");
+  EI_REQUIRE(scale > 0.f, "attention_prefill: the scale must be positive");
+  const AttnExtra extra{chunk, slopes, sinks};
+  return prefill_launch(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
+                        page_table, table_width, out, nq, nkv, D, window, scale, key_ways,
+                        pair_items, &extra, stream);
 }
 
 // Whether the decode kernel of this file takes a head size and group ratio.
@@ -1022,7 +1127,9 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
                          const int32_t* page_table, int table_width, void* out, float* part_o,
                          float* part_ml, int rows, int nq, int nkv, int D, int window,
                          float scale, int n_splits, int waves, int heads, const int32_t* longest,
-                         const DecodePrep* prep, hipStream_t stream) {
+                         const DecodePrep* prep, hipStream_t stream,
+                         const AttnExtra* extra = nullptr) {
+  EI_REQUIRE(!(prep && extra), "attention_decode: the fused projection has no extended form");
   EI_REQUIRE(rows > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad head counts");
   EI_REQUIRE(waves == 4 || waves == 8 || waves == 16,
              "attention_decode: a block has 4, 8 or 16 waves");
@@ -1054,16 +1161,24 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
   const bf16_t* vv = static_cast<const bf16_t*>(v_pages);
   bf16_t* oo = static_cast<bf16_t*>(out);
   const DecodePrep none{};
+  const AttnExtra plain{0, nullptr, nullptr};
 #define EI_DECODE(DD, GG)                                                                     \
   do {                                                                                        \
     if (prep)                                                                                 \
-      launch_decode<DD, GG, true>(grid, stream, qq, kk, vv, row_pos, row_seq, page_table,     \
-                                  table_width, oo, part_o, part_ml, nq, nkv, head_blocks,     \
-                                  window, scale, n_splits, waves, longest, *prep);            \
+      launch_decode<DD, GG, true, false>(grid, stream, qq, kk, vv, row_pos, row_seq,          \
+                                         page_table, table_width, oo, part_o, part_ml, nq,    \
+                                         nkv, head_blocks, window, scale, n_splits, waves,    \
+                                         longest, *prep, plain);                              \
+    else if (extra)                                                                           \
+      launch_decode<DD, GG, false, true>(grid, stream, qq, kk, vv, row_pos, row_seq,          \
+                                         page_table, table_width, oo, part_o, part_ml, nq,    \
+                                         nkv, head_blocks, window, scale, n_splits, waves,    \
+                                         longest, none, *extra);                              \
     else                                                                                      \
-      launch_decode<DD, GG, false>(grid, stream, qq, kk, vv, row_pos, row_seq, page_table,    \
-                                   table_width, oo, part_o, part_ml, nq, nkv, head_blocks,    \
-                                   window, scale, n_splits, waves, longest, none);            \
+      launch_decode<DD, GG, false, false>(grid, stream, qq, kk, vv, row_pos, row_seq,         \
+                                          page_table, table_width, oo, part_o, part_ml, nq,   \
+                                          nkv, head_blocks, window, scale, n_splits, waves,   \
+                                          longest, none, plain);                              \
   } while (0)
 #define EI_DECODE_G(DD)            \
   switch (GB) {                    \
@@ -1112,6 +1227,24 @@ extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, cons
   return decode_launch(q, k_pages, v_pages, row_pos, row_seq, page_table, table_width, out,
                        part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, heads,
                        longest, nullptr, stream);
+}
+
+// The same with the options of `AttnExtra`: chunk (0: none), slopes and sinks (float32 [nq] on
+// the device, or null).
+extern "C" int ei_attention_decode_mfma_ext(const void* q, const void* k_pages,
+                                            const void* v_pages, const int32_t* row_pos,
+                                            const int32_t* row_seq, const int32_t* page_table,
+                                            int table_width, void* out, float* part_o,
+                                            float* part_ml, int rows, int nq, int nkv, int D,
+                                            int window, float scale, int n_splits, int waves,
+                                            int heads, const int32_t* longest, int chunk,
+                                            const float* slopes, const float* sinks,
+                                            hipStream_t stream) {
+  EI_REQUIRE(chunk >= 0, "attention_decode: negative chunk");
+  const AttnExtra extra{chunk, slopes, sinks};
+  return decode_launch(q, k_pages, v_pages, row_pos, row_seq, page_table, table_width, out,
+                       part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, heads,
+                       longest, nullptr, stream, &extra);
 }
 
 // The same from the fused projection instead of q: qkv float32 [nsplit][rows, (nq + 2 nkv) * D]

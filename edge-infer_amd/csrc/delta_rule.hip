@@ -33,7 +33,15 @@ constexpr int kMaxTaps = 32;
 template <typename TI>
 __device__ __forceinline__ float slice_sum(const TI* p, int nsplit, size_t stride) {
   float x = 0.f;
-  for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TI>(p[s * stride]);
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {        // eight slices per trip to memory, added in order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s0 + u < nsplit) v[u] = ei::to_f32<TI>(p[(s0 + u) * stride]);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s0 + u < nsplit) x += v[u];
+  }
   return x;
 }
 
@@ -146,7 +154,10 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
   __shared__ __attribute__((aligned(16))) float q_s[TILE][DP];
   __shared__ __attribute__((aligned(16))) float k_s[TILE][DP];
   __shared__ float v_s[TILE][CB];
-  __shared__ float beta_s[kTile], decay_s[kTile], qf_s[kTile], kf_s[kTile];
+  // per token: decay g, the factor that makes k a unit vector, beta times that factor, and
+  // the factor of q (unit vector times q_scale)
+  __shared__ __attribute__((aligned(16))) float4 coef_s[TILE];
+  __shared__ float beta_s[TILE], decay_s[TILE];
 
   const int seq = blockIdx.x;
   const int count = seq_count[seq];
@@ -162,9 +173,27 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
 
   float* mine = state + static_cast<size_t>(seq_slot[seq]) * state_stride +
                 (static_cast<size_t>(head) * DV + (col_ok ? col : 0)) * D + i0;
+  // (D a multiple of 4: the rows a thread owns are whole 16-byte pieces, inside S or outside)
+  const bool wide = D % 4 == 0;
   float s[kOwn];
 #pragma unroll
-  for (int m = 0; m < kOwn; ++m) s[m] = (col_ok && i0 + m < D) ? mine[m] : 0.f;
+  for (int m = 0; m < kOwn; ++m) s[m] = 0.f;
+  if (col_ok) {
+    if (wide) {
+      if (i0 < D) {
+        const float4 a = *reinterpret_cast<const float4*>(mine);
+        s[0] = a.x; s[1] = a.y; s[2] = a.z; s[3] = a.w;
+      }
+      if (i0 + 4 < D) {
+        const float4 a = *reinterpret_cast<const float4*>(mine + 4);
+        s[4] = a.x; s[5] = a.y; s[6] = a.z; s[7] = a.w;
+      }
+    } else {
+#pragma unroll
+      for (int m = 0; m < kOwn; ++m)
+        if (i0 + m < D) s[m] = mine[m];
+    }
+  }
   const float rate = expf(a_log[head]), shift = dt_bias[head];
 
   for (int t0 = 0; t0 < count; t0 += TILE) {
@@ -201,45 +230,61 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
       q_sq = group_sum<8>(q_sq);
       k_sq = group_sum<8>(k_sq);
       if (tt < nt && sub == 0) {
-        qf_s[tt] = q_scale / sqrtf(q_sq + unit_eps);
-        kf_s[tt] = 1.0f / sqrtf(k_sq + unit_eps);
+        const float kf = 1.0f / sqrtf(k_sq + unit_eps);
+        coef_s[tt] = make_float4(decay_s[tt], kf, beta_s[tt] * kf, q_scale / sqrtf(q_sq + unit_eps));
       }
     }
     __syncthreads();
+    // the walk: what token tt + 1 needs is read from LDS while token tt is computed
+    float4 ka = *reinterpret_cast<const float4*>(&k_s[0][i0]);
+    float4 kb = *reinterpret_cast<const float4*>(&k_s[0][i0 + 4]);
+    float4 qa = *reinterpret_cast<const float4*>(&q_s[0][i0]);
+    float4 qb = *reinterpret_cast<const float4*>(&q_s[0][i0 + 4]);
+    float4 cf = coef_s[0];
+    float vv = v_s[0][col_in_block];
     for (int tt = 0; tt < nt; ++tt) {
-      const float g = decay_s[tt], kf = kf_s[tt];
-      float kv[kOwn], qv[kOwn];
-      *reinterpret_cast<float4*>(kv) = *reinterpret_cast<const float4*>(&k_s[tt][i0]);
-      *reinterpret_cast<float4*>(kv + 4) = *reinterpret_cast<const float4*>(&k_s[tt][i0 + 4]);
-      *reinterpret_cast<float4*>(qv) = *reinterpret_cast<const float4*>(&q_s[tt][i0]);
-      *reinterpret_cast<float4*>(qv + 4) = *reinterpret_cast<const float4*>(&q_s[tt][i0 + 4]);
+      const float kv[kOwn] = {ka.x, ka.y, ka.z, ka.w, kb.x, kb.y, kb.z, kb.w};
+      const float qv[kOwn] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+      const float g = cf.x, kf = cf.y, bk = cf.z, qf = cf.w, v_now = vv;
+      const int nx = tt + 1 < nt ? tt + 1 : tt;
+      ka = *reinterpret_cast<const float4*>(&k_s[nx][i0]);
+      kb = *reinterpret_cast<const float4*>(&k_s[nx][i0 + 4]);
+      qa = *reinterpret_cast<const float4*>(&q_s[nx][i0]);
+      qb = *reinterpret_cast<const float4*>(&q_s[nx][i0 + 4]);
+      cf = coef_s[nx];
+      vv = v_s[nx][col_in_block];
       float seen0 = 0.f, seen1 = 0.f;
 #pragma unroll
       for (int m = 0; m < kOwn; m += 2) {
         s[m] *= g;
         s[m + 1] *= g;
-        seen0 += s[m] * kv[m];
-        seen1 += s[m + 1] * kv[m + 1];
+        seen0 = fmaf(s[m], kv[m], seen0);
+        seen1 = fmaf(s[m + 1], kv[m + 1], seen1);
       }
       const float seen = group_sum<L>(seen0 + seen1) * kf;       // (S^T k)[col], k a unit vector
-      const float u = beta_s[tt] * (v_s[tt][col_in_block] - seen) * kf;
+      const float u = bk * (v_now - seen);                       // beta (v - S^T k), times k's factor
       float o0 = 0.f, o1 = 0.f;
 #pragma unroll
       for (int m = 0; m < kOwn; m += 2) {
-        s[m] += kv[m] * u;
-        s[m + 1] += kv[m + 1] * u;
-        o0 += s[m] * qv[m];
-        o1 += s[m + 1] * qv[m + 1];
+        s[m] = fmaf(kv[m], u, s[m]);
+        s[m + 1] = fmaf(kv[m + 1], u, s[m + 1]);
+        o0 = fmaf(s[m], qv[m], o0);
+        o1 = fmaf(s[m + 1], qv[m + 1], o1);
       }
-      const float o = group_sum<L>(o0 + o1) * qf_s[tt];
+      const float o = group_sum<L>(o0 + o1) * qf;
       if (part == 0 && col_ok)
         o_raw[static_cast<size_t>(row0 + t0 + tt) * VW + head * DV + col] = o;
     }
   }
   if (col_ok) {
+    if (wide) {
+      if (i0 < D) *reinterpret_cast<float4*>(mine) = make_float4(s[0], s[1], s[2], s[3]);
+      if (i0 + 4 < D) *reinterpret_cast<float4*>(mine + 4) = make_float4(s[4], s[5], s[6], s[7]);
+    } else {
 #pragma unroll
-    for (int m = 0; m < kOwn; ++m)
-      if (i0 + m < D) mine[m] = s[m];
+      for (int m = 0; m < kOwn; ++m)
+        if (i0 + m < D) mine[m] = s[m];
+    }
   }
 }
 

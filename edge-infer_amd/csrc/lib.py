@@ -78,6 +78,14 @@ _SIGNATURES = {
                                      c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                      c_int, c_int, c_float, c_int, c_int, c_int, c_void_p,
                                      c_void_p],
+        "ei_attention_prefill_mfma_ext": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
+                                          c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                          c_int, c_void_p, c_void_p, c_void_p],
+        "ei_attention_decode_mfma_ext": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                         c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                         c_void_p, c_int, c_void_p, c_void_p, c_void_p],
         "ei_attention_decode_mfma_fused": [c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_float,
                                            c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -499,14 +507,16 @@ def attention_prefill_mfma_positions(group: int, key_ways: int = 1) -> int:
 
 def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
                            page_table, out, n_heads, n_kv_heads, head_dim, window=None,
-                           scale=None, key_ways=1, pair_items=True, largest_item=None) -> None:
+                           scale=None, key_ways=1, pair_items=True, largest_item=None,
+                           chunk=None, slopes=None, sinks=None) -> None:
     """bfloat16 prefill attention on the matrix cores; an item holds up to
     `attention_prefill_mfma_positions(group, key_ways)` positions of one sequence.
     pair_items: with enough items a block may take item i and then item n_items - 1 - i
     (equal work a block where the items are those of one prompt, longest first).
     largest_item: the most positions any item holds, from the host's copy of the list (the
     kernel gives a block's waves fixed rows of an item and would leave the rows of a larger
-    one out); None: looked up from `item_npos` on the device, which waits for the device."""
+    one out); None: looked up from `item_npos` on the device, which waits for the device.
+    chunk, slopes, sinks: as for `attention` (any of them takes the kernel's extended form)."""
     lib = library("attention_mfma")
     n = q.shape[0]
     capacity = attention_prefill_mfma_positions(n_heads // max(1, n_kv_heads), key_ways)
@@ -527,15 +537,29 @@ def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, 
         raise KernelError("attention_prefill: work item arrays shorter than n_items")
     if scale is None:
         scale = head_dim ** -0.5
-    status = lib.ei_attention_prefill_mfma(
+    common = (
         _gpu(q, "q", torch.bfloat16), _gpu(k_pages, "k_pages", torch.bfloat16),
         _gpu(v_pages, "v_pages", torch.bfloat16), _gpu(item_seq, "item_seq", torch.int32),
         _gpu(item_row0, "item_row0", torch.int32), _gpu(item_npos, "item_npos", torch.int32),
         n_items, _gpu(row_pos, "row_pos", torch.int32),
         _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
         _gpu(out, "out", torch.bfloat16), n_heads, n_kv_heads, head_dim, int(window or 0),
-        float(scale), int(key_ways), int(bool(pair_items)), _stream())
+        float(scale), int(key_ways), int(bool(pair_items)))
+    if chunk or slopes is not None or sinks is not None:
+        status = lib.ei_attention_prefill_mfma_ext(*common, *_attention_extras(
+            chunk, slopes, sinks, n_heads), _stream())
+    else:
+        status = lib.ei_attention_prefill_mfma(*common, _stream())
     _check(lib, status, "attention_prefill")
+
+
+def _attention_extras(chunk, slopes, sinks, n_heads):
+    """(chunk, slopes pointer, sinks pointer) for the extended forms of the matrix-core kernels."""
+    for name, per_head in (("slopes", slopes), ("sinks", sinks)):
+        if per_head is not None and per_head.numel() != n_heads:
+            raise KernelError(f"attention: {name} must have one value per query head")
+    return (int(chunk or 0), None if slopes is None else _gpu(slopes, "slopes", torch.float32),
+            None if sinks is None else _gpu(sinks, "sinks", torch.float32))
 
 
 class DecodeProjection:
@@ -552,7 +576,8 @@ class DecodeProjection:
 
 def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out, n_heads,
                           n_kv_heads, head_dim, window=None, scale=None, n_splits=1, part_o=None,
-                          part_ml=None, waves=4, longest=None, heads=0) -> None:
+                          part_ml=None, waves=4, longest=None, heads=0, chunk=None, slopes=None,
+                          sinks=None) -> None:
     """bfloat16 decode attention on the matrix cores: one query row per sequence.  `waves`
     (4, 8 or 16) of a block share its key range tile by tile; more suit fewer sequences (few
     blocks), whose ranges then need fewer slices or none.  `heads` (a power of two, or 0 for
@@ -561,10 +586,14 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
     device): the most tokens a sequence of the step holds; every sequence's range is then
     cut into slices of the longest one's share, so that unequal lengths give equal blocks.
     `q` is the queries [rows, heads * head_dim], or a `DecodeProjection`: the kernel then does
-    the work of `qk_norm_rope_store` for its rows as well."""
+    the work of `qk_norm_rope_store` for its rows as well.  chunk, slopes, sinks: as for
+    `attention` (any of them takes the kernel's extended form, which the fused one lacks)."""
     lib = library("attention_mfma")
     n = out.shape[0]
     fused = isinstance(q, DecodeProjection)
+    extended = bool(chunk) or slopes is not None or sinks is not None
+    if fused and extended:
+        raise KernelError("attention_decode: the fused projection has no extended form")
     if tuple(out.shape) != (n, n_heads * head_dim) or (not fused and tuple(q.shape) != tuple(out.shape)):
         raise KernelError("attention_decode: q and out must be [rows, heads * head_dim]")
     if fused:
@@ -606,7 +635,7 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
             _stream())
         _check(lib, status, "attention_decode")
         return
-    status = lib.ei_attention_decode_mfma(
+    common = (
         _gpu(q, "q", torch.bfloat16), _gpu(k_pages, "k_pages", torch.bfloat16),
         _gpu(v_pages, "v_pages", torch.bfloat16), _gpu(row_pos, "row_pos", torch.int32),
         _gpu(row_seq, "row_seq", torch.int32), _gpu(page_table, "page_table", torch.int32),
@@ -614,7 +643,12 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
         None if part_o is None else _gpu(part_o, "part_o", torch.float32),
         None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
         n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, int(waves), int(heads),
-        None if longest is None else _gpu(longest, "longest", torch.int32), _stream())
+        None if longest is None else _gpu(longest, "longest", torch.int32))
+    if extended:
+        status = lib.ei_attention_decode_mfma_ext(*common, *_attention_extras(
+            chunk, slopes, sinks, n_heads), _stream())
+    else:
+        status = lib.ei_attention_decode_mfma(*common, _stream())
     _check(lib, status, "attention_decode")
 
 

@@ -373,7 +373,15 @@ __global__ void projection_norm_store_kernel(
   float q_sq = 0.f, k_sq = 0.f;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float x = 0.f;
-    for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TI>(src[s * split_stride + i]);
+    for (int s0 = 0; s0 < nsplit; s0 += 8) {      // eight slices per trip to memory
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < nsplit) v[u] = ei::to_f32<TI>(src[(s0 + u) * split_stride + i]);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < nsplit) x += v[u];
+    }
     row_values[i] = x;
     if (i < QW) q_sq += x * x;
     else if (i < QW + KW) k_sq += x * x;

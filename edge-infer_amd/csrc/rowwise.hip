@@ -419,6 +419,63 @@ __global__ void norm_add_kernel(float* __restrict__ residual, const TD* __restri
   }
 }
 
+// The same for widths that are a multiple of 4: 16-byte accesses, the row kept in registers,
+// the slices' loads issued eight at a time (they are added in slice order).
+template <typename TD, typename TO, int CHUNKS>
+__global__ void norm_add_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                    int nsplit, size_t split_stride,
+                                    const float* __restrict__ weight, float eps,
+                                    TO* __restrict__ cast_out, int H) {
+  __shared__ float scratch[16];
+  const size_t base = static_cast<size_t>(blockIdx.x) * H;
+  const int quads = H / 4;
+  float w[CHUNKS][4], r[CHUNKS][4], x[CHUNKS][4];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) {
+      Vec4<float>::load(weight + qd * 4, w[k]);
+      Vec4<float>::load(residual + base + qd * 4, r[k]);
+    }
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    x[k][0] = x[k][1] = x[k][2] = x[k][3] = 0.f;
+    if (qd < quads) {
+      const TD* d = delta + base + qd * 4;
+      for (int s0 = 0; s0 < nsplit; s0 += 8) {
+        float v[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) Vec4<TD>::load(d + (s0 + u) * split_stride, v[u]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) x[k][i] += v[u][i];
+          }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sum += x[k][i] * x[k][i];
+    }
+  }
+  const float total = ei::block_sum(sum, scratch);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(H) + eps);
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) {
+      float y[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = r[k][i] + (x[k][i] * inv) * w[k][i];
+      Vec4<float>::store(residual + base + qd * 4, y);
+      if (cast_out) Vec4<TO>::store(cast_out + base + qd * 4, y);
+    }
+  }
+}
+
 template <typename TO>
 __global__ void cast_rows_kernel(const float* __restrict__ in, TO* __restrict__ out, size_t n) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -448,7 +505,15 @@ __global__ void activation_kernel(const TI* __restrict__ in, int nsplit, size_t 
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   for (size_t i = start; i < n; i += step) {
     float x = 0.f;
-    for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TI>(in[s * split_stride + i]);
+    for (int s0 = 0; s0 < nsplit; s0 += 8) {      // eight slices per trip to memory
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < nsplit) v[u] = ei::to_f32<TI>(in[(s0 + u) * split_stride + i]);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < nsplit) x += v[u];
+    }
     out[i] = ei::from_f32<TO>(activate(x, kind));
   }
 }
@@ -467,15 +532,32 @@ extern "C" int ei_norm_add(float* residual, const void* delta, int delta_dtype, 
   const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
   const size_t lds = static_cast<size_t>(H) * sizeof(float);
   const size_t ss = static_cast<size_t>(split_stride);
+  const bool vec = H % 4 == 0 && ss % 4 == 0;
+  const int quads = H / 4;
+  // few rows: up to 1024 threads a row, so that many loads are in flight; many rows: 256
+  const int most = N >= 512 && quads <= 4 * 256 ? 256 : 1024;
+  int vthreads = (quads + EI_WAVE - 1) / EI_WAVE * EI_WAVE;
+  if (vthreads > most) vthreads = most;
+  const int chunks = vec ? (quads + vthreads - 1) / vthreads : 0;      // 1..4 for H <= 16384
+#define EI_NORM_ADD_VEC(TD, TO, C)                                                               \
+  norm_add_vec_kernel<TD, TO, C><<<N, vthreads, 0, stream>>>(                                    \
+      residual, static_cast<const TD*>(delta), nsplit, ss, weight, eps, static_cast<TO*>(cast_out), H)
 #define EI_NORM_ADD(TD, TO)                                                                      \
-  norm_add_kernel<TD, TO><<<N, threads, lds, stream>>>(residual, static_cast<const TD*>(delta),  \
-                                                       nsplit, ss, weight, eps,                  \
-                                                       static_cast<TO*>(cast_out), H)
+  do {                                                                                           \
+    if (chunks == 1) EI_NORM_ADD_VEC(TD, TO, 1);                                                 \
+    else if (chunks == 2) EI_NORM_ADD_VEC(TD, TO, 2);                                            \
+    else if (chunks >= 3) EI_NORM_ADD_VEC(TD, TO, 4);                                            \
+    else                                                                                         \
+      norm_add_kernel<TD, TO><<<N, threads, lds, stream>>>(                                      \
+          residual, static_cast<const TD*>(delta), nsplit, ss, weight, eps,                      \
+          static_cast<TO*>(cast_out), H);                                                        \
+  } while (0)
   if (delta_dtype == EI_F32 && (out_dtype == EI_F32 || !cast_out)) EI_NORM_ADD(float, float);
   else if (delta_dtype == EI_F32 && out_dtype == EI_BF16) EI_NORM_ADD(float, bf16_t);
   else if (delta_dtype == EI_BF16 && (out_dtype == EI_BF16 || !cast_out)) EI_NORM_ADD(bf16_t, bf16_t);
   else EI_REQUIRE(false, "norm_add: unsupported dtype combination");
 #undef EI_NORM_ADD
+#undef EI_NORM_ADD_VEC
   EI_LAUNCH_CHECK();
 }
 

@@ -8,7 +8,8 @@ become one [Q + 2 KV, H] matrix when the part is built: each output element is
 still the same dot product.  Each projection may have a bias
 (runtime/include/models/qwen3_model.hpp:386-395: taken if the checkpoint holds it).
 
-Options of the spec beyond that decoder (any of them sends the mixer down the generic
+Options of the spec beyond that decoder (the matrix-core kernels have an extended form for
+chunks, slopes and the sink; values of another width than the keys go down the generic
 float32-arithmetic kernels): values narrower or wider than keys (`value_dim`), one RMS norm
 over the whole q and the whole k projection instead of one per head (`qk_norm_scope =
 "projection"`), visibility in blocks of `chunk` positions counted from the sequence's start,
@@ -101,7 +102,7 @@ class Attention:
         """What this part will run, so that a model can have it compiled ahead of its first
         step."""
         group = spec.n_heads // max(1, spec.n_kv_heads)
-        fast = (dtype == torch.bfloat16 and not spec.extended
+        fast = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim
                 and lib.attention_decode_mfma_supported(spec.head_dim, group))
         return ("rope_store", "attention_mfma" if fast else "attention_generic",
                 *Linear.kernel_libraries(dtype))
@@ -166,10 +167,13 @@ class Attention:
             self.slopes = torch.pow(2.0, exponent).to(device=device, dtype=torch.float32).contiguous()
         if spec.sink:
             self.sinks = params["sink"].to(device=device, dtype=torch.float32).contiguous()
-        # the matrix-core kernels take bfloat16 with head sizes 64 and 128 and none of the
-        # options beyond rotary, windowed attention; every other case runs the generic kernel
-        self.matrix_cores = (dtype == torch.bfloat16 and not spec.extended and
+        # the matrix-core kernels take bfloat16 with head sizes 64 and 128 and values as wide
+        # as the keys; every other case runs the generic kernel
+        self.matrix_cores = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
+        # chunk, slopes, sink: what the kernels take beyond a window
+        self.extras = dict(chunk=spec.chunk, slopes=self.slopes, sinks=self.sinks)
+        self.has_extras = spec.chunk is not None or self.slopes is not None or self.sinks is not None
         self.compute_units = lib.compute_units(device)     # the chip's size, for launch plans
         self._decode_launches = {}     # (sequences, pages of context) -> decode_launch's answer
 
@@ -304,7 +308,7 @@ class Attention:
         page_table = meta.page_table(group_index)
         qkv = self.qkv.forward(ctx, x, "attn.qkv")
         if (ctx.decode and self.matrix_cores and FUSED_DECODE and qkv.dim() == 3
-                and qkv.dtype == torch.float32):
+                and qkv.dtype == torch.float32 and not self.whole_store and not self.has_extras):
             # the decode kernel norms, rotates and stores for its rows itself: one launch less
             q = lib.DecodeProjection(qkv, self.q_norm, self.k_norm, spec.qk_norm_eps,
                                      self.position.table, entry.writes_cache)
@@ -321,7 +325,7 @@ class Attention:
                 meta.row_pos, meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads,
                 spec.n_kv_heads, spec.head_dim, write_cache=entry.writes_cache)
         out = ctx.buffer("attn.out", (n, spec.out_width))
-        more = dict(value_dim=spec.v_dim, chunk=spec.chunk, slopes=self.slopes, sinks=self.sinks)
+        more = dict(value_dim=spec.v_dim, **self.extras)
         part_o = part_ml = None
         if ctx.decode:
             splits, waves, heads = self._decode_launch_for(ctx.n_seqs, ctx.context_bound)
@@ -335,7 +339,8 @@ class Attention:
                                           page_table, out, spec.n_heads, spec.n_kv_heads,
                                           spec.head_dim, window=spec.window, scale=self.scale,
                                           n_splits=splits, part_o=part_o, part_ml=part_ml,
-                                          waves=waves, longest=meta.longest, heads=heads)
+                                          waves=waves, longest=meta.longest, heads=heads,
+                                          **self.extras)
             else:
                 item_seq, item_row0, item_npos, n_items = self._items(ctx, "attention.decode_items")
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
@@ -358,7 +363,7 @@ class Attention:
                                            spec.n_kv_heads, spec.head_dim, window=spec.window,
                                            scale=self.scale, key_ways=key_ways,
                                            pair_items=len({(seq.start, seq.count) for seq in ctx.sequences}) == 1,
-                                           largest_item=largest)
+                                           largest_item=largest, **self.extras)
             else:
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,

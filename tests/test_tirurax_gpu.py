@@ -15,8 +15,8 @@ from tirurax_helpers import CONFIGS, ids, sharp_weights, write_folder
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-NAMES = ["A", "B"]
-LENGTHS = {"A": [150, 1, 49, 75], "B": [210, 2, 101, 64]}
+NAMES = ["A", "B", "C"]
+LENGTHS = {"A": [150, 1, 49, 75], "B": [210, 2, 101, 64], "C": [330, 3, 130, 65]}
 # bfloat16 engine against the float64 oracle on these order-one weights: root-mean-square
 # error relative to the logits' root-mean-square, and largest error relative to the
 # largest logit (a recurrent state and several renormalised sublayers round more often
@@ -122,7 +122,7 @@ def test_batches_of_unequal_requests_with_slots_and_pages_used_again(models, ref
     import edge_infer_amd as ei
     requests, refs = requests_for(name), references[name]
     tail = 20
-    session = ei.Session(models(name, dtype), max_tokens=64 * 9, max_seqs=4)
+    session = ei.Session(models(name, dtype), max_tokens=64 * 12, max_seqs=4)
     for batch in ([0, 1, 2, 3], [3, 2, 0], [1, 0, 3, 2]):
         slots = {i: session.begin() for i in batch}
         cuts = {i: max(1, len(requests[i]) - tail) for i in batch}
@@ -168,7 +168,7 @@ def test_long_decoding_from_the_first_token(models, weights, name, dtype):
         assert (name, dtype) == ("B", "bfloat16")
 
 
-@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("name", ["A", "B"])
 def test_a_token_far_back_shows(tmp_path, name):
     """Delta layers that forget slowly: two prompts that differ in their third token alone
     still differ at position 400, by far more than the tolerance, and the engine follows the
@@ -197,7 +197,7 @@ def test_a_token_far_back_shows(tmp_path, name):
         session.end(slot)
 
 
-@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("name", ["A", "B"])
 def test_greedy_generation_through_the_entry_point(models, weights, name):
     """`Session.generate_batch` (the scheduler, sampler and step function together) gives the
     oracle's greedy tokens in float32."""

@@ -156,17 +156,21 @@ def test_attention_options_alone(variant):
                          f"{variant}: token {t}")
 
 
+@pytest.mark.parametrize("head_dim, dtype", [(32, "float32"), (64, "bfloat16"), (128, "bfloat16")])
 @pytest.mark.parametrize("decoded", [False, True])
 @pytest.mark.parametrize("where", ["just outside", "just inside", "far inside", "nowhere"])
-def test_a_key_that_stands_out_at_a_chunks_edge(where, decoded):
+def test_a_key_that_stands_out_at_a_chunks_edge(where, decoded, head_dim, dtype):
     """Query and key projections are made equal and read only the first half of an input row
     (the values read the other half), so a key whose row shares that half with the query's
     scores as high as the query's own key and far above every other (32 against a few units).
     Put just outside the query's chunk it must change nothing; just inside (37 positions
     back, which the distance term of the second head hardly lowers), or next to the query, it
     takes up to half the weight for a value of its own.  The query is the last row of a
-    prompt, or a token decoded alone."""
-    mixer = attention_spec(n_heads=2, n_kv_heads=2, head_dim=32, value_dim=8, chunk=50)
+    prompt, or a token decoded alone.  In bfloat16 with head sizes 64 and 128 the matrix-core
+    kernels run (values as wide as the keys; the scale keeps the score that stands out at 32)."""
+    value_dim = 8 if dtype == "float32" else head_dim
+    mixer = attention_spec(n_heads=2, n_kv_heads=2, head_dim=head_dim, value_dim=value_dim,
+                           chunk=50, scale=32.0 / head_dim)
     spec = one_layer(mixer)
     params = params_for(spec, 5)
     half = HIDDEN // 2
@@ -175,8 +179,9 @@ def test_a_key_that_stands_out_at_a_chunks_edge(where, decoded):
     params["layers.0.mixer.k_proj.weight"] = params["layers.0.mixer.q_proj.weight"].clone()
     params["layers.0.mixer.k_proj.bias"] = params["layers.0.mixer.q_proj.bias"].clone()
     params["layers.0.mixer.k_norm.weight"] = params["layers.0.mixer.q_norm.weight"].clone()
-    model, session = session_for(spec, params)
+    model, session = session_for(spec, params, dtype)
     part = model.layers[0].mixer
+    assert part.matrix_cores == (dtype == "bfloat16")
     torch.manual_seed(2)
     query = 137                                   # its chunk is 100..149
     x = torch.randn(query + 1, HIDDEN)
@@ -188,12 +193,17 @@ def test_a_key_that_stands_out_at_a_chunks_edge(where, decoded):
     moved = (expected - plainly).abs().max().item() / plainly.abs().max().item()
     assert (moved > 0.1) == (where in ("just inside", "far inside")), moved
     slot = session.begin()
+    x = x.to(model.dtype)
     if decoded:
         run_part(session, part, [(slot, 0, x[:query])])
         out = run_part(session, part, [(slot, query, x[query:])])[0]
     else:
         out = run_part(session, part, [(slot, 0, x)])[query]
-    assert_close_f32(out, expected, f"key {where}")
+    if dtype == "float32":
+        assert_close_f32(out, expected, f"key {where}")
+    else:       # bfloat16 queries, keys and probabilities: a few per cent of the largest output
+        error = (out.double().cpu() - expected).abs().max() / expected.abs().max()
+        assert error < 0.04, f"key {where}: {error:.3f}"
 
 
 def test_the_sink_and_the_slopes_count():

@@ -3,7 +3,9 @@
 The configurations differ from each other in every size and option: key and value head
 sizes that differ, group ratios 1, 3 and 4, chunks that are no multiple of the cache's page
 of 64 tokens (and none at all), 1 to 5 convolution taps, key sizes that are no multiple of
-8 and above 128, layers without a feed-forward, both layer kinds first.  The weights are
+8 and above 128, layers without a feed-forward, both layer kinds first, and (C) attention
+with head sizes 64 and 128 and values as wide as keys, which in bfloat16 runs on the
+matrix-core kernels.  The weights are
 drawn so that signals are of order one (N(0, 0.02) matrices would make every softmax flat
 and every state tiny, and hide a wrong key or a lost state); they are rounded to bfloat16,
 so that both precisions and the oracle see the same numbers.
@@ -34,7 +36,12 @@ CONFIG_A = {"architecture": "Tirurax", "vocab": 211, "width": 64, "norm": {"eps"
 CONFIG_B = {"architecture": "Tirurax", "vocab": 97, "width": 96, "norm": {"eps": 1e-6},
             "layers": [delta(2, 1, 40, 20, 5, 128), attention(3, 3, 8, 48, 0.5, 100, None),
                        delta(1, 1, 160, 12, 1, 64), attention(8, 2, 16, 16, 0.25, 7, 40)]}
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B}
+# head sizes 64 and 128 with values as wide as keys: what the matrix-core attention kernels take
+CONFIG_C = {"architecture": "Tirurax", "vocab": 150, "width": 128, "norm": {"eps": 1e-6},
+            "layers": [attention(4, 2, 64, 64, 0.15, 48, 160), delta(2, 2, 32, 64, 4, 96),
+                       attention(2, 1, 128, 128, 0.1, 200, None),
+                       attention(8, 2, 64, 64, 0.125, None, 64)]}
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
 
 
 def tensor_shapes(cfg):
