@@ -29,6 +29,7 @@ constexpr int kThreads = 256;
 constexpr int kTile = 32;        // most tokens of a sequence that delta_rule stages in LDS at a time
 constexpr int kOwn = 8;          // rows of a column of S that one thread owns
 constexpr int kMaxTaps = 32;
+constexpr int kFewTaps = 8;      // up to so many taps a thread keeps a channel's inputs in registers
 
 template <typename TI>
 __device__ __forceinline__ float slice_sum(const TI* p, int nsplit, size_t stride) {
@@ -52,6 +53,8 @@ __device__ __forceinline__ float softplus_f32(float x) {
 }
 
 // proj: [nsplit][N, WP]; the convolved channels are its first C columns.  conv_w: [C, J].
+// new_tail_state (the state again, or null): a step in which every sequence brings one row
+// may have the tails renewed here (up to kFewTaps taps), which saves the launch of delta_tail.
 // The tail of a sequence (its last J - 1 inputs before this step, oldest first) lies at
 // state + slot * state_stride + tail_offset as [J - 1, C].
 template <typename TI>
@@ -62,58 +65,72 @@ __global__ void delta_conv_kernel(const TI* __restrict__ proj, int nsplit, size_
                                   const int32_t* __restrict__ row_seq,
                                   const int32_t* __restrict__ seq_slot,
                                   const int32_t* __restrict__ seq_start, float* __restrict__ out,
-                                  size_t total, int C) {
-  const size_t first = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
-  for (size_t idx = first; idx < total; idx += step) {
-    const size_t row = idx / C;
-    const int c = static_cast<int>(idx % C);
-    const int seq = row_seq[row];
-    if (seq < 0) continue;
-    const int pos = row_pos[row], start = seq_start[seq];
-    const float* tail = state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
-    float acc = 0.f;
-    for (int j = 0; j < J; ++j) {
-      const int back = J - 1 - j;
-      const int p = pos - back;
-      float x = 0.f;
-      if (p >= start)
-        x = slice_sum(proj + (row - back) * WP + c, nsplit, split_stride);
-      else if (p >= 0)
-        x = tail[static_cast<size_t>(p - start + J - 1) * C + c];
-      acc += conv_w[static_cast<size_t>(c) * J + j] * x;
+                                  int C, float* __restrict__ new_tail_state) {
+  const size_t row = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int seq = row_seq[row];
+  if (seq < 0 || c >= C) return;
+  const int pos = row_pos[row], start = seq_start[seq];
+  const float* tail = state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+  auto input = [&](int j) {                  // the input that tap j multiplies
+    const int back = J - 1 - j;
+    const int p = pos - back;
+    if (p >= start) return slice_sum(proj + (row - back) * WP + c, nsplit, split_stride);
+    if (p >= 0) return tail[static_cast<size_t>(p - start + J - 1) * C + c];
+    return 0.f;
+  };
+  float acc = 0.f;
+  if (J <= kFewTaps) {                       // every input is asked for before the first is used
+    float x[kFewTaps];
+#pragma unroll
+    for (int j = 0; j < kFewTaps; ++j) x[j] = j < J ? input(j) : 0.f;
+#pragma unroll
+    for (int j = 0; j < kFewTaps; ++j)
+      if (j < J) acc += conv_w[static_cast<size_t>(c) * J + j] * x[j];
+    if (new_tail_state) {
+      // every sequence brings this one row (the caller says so): the thread is the only
+      // reader of its channel's tail, and the new tail is the inputs it holds, moved by one
+      float* to = new_tail_state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+#pragma unroll
+      for (int j = 1; j < kFewTaps; ++j)
+        if (j < J) to[static_cast<size_t>(j - 1) * C + c] = x[j];
     }
-    out[idx] = silu_f32(acc);
+  } else {
+    for (int j = 0; j < J; ++j) acc += conv_w[static_cast<size_t>(c) * J + j] * input(j);
   }
+  out[row * C + c] = silu_f32(acc);
 }
 
-// The thread of a sequence's last row of the step writes the sequence's new tail for its
-// channel: the inputs of the last J - 1 positions, from this step's rows or, where the step
-// brought fewer, from the old tail (read before anything is written).
+// A thread writes a sequence's new tail for its channel: the inputs of the last J - 1
+// positions, from this step's rows or, where the step brought fewer, from the old tail (read
+// before anything is written).
 template <typename TI>
 __global__ void delta_tail_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                                   int WP, int J, float* __restrict__ state, size_t state_stride,
-                                  size_t tail_offset, const int32_t* __restrict__ row_pos,
-                                  const int32_t* __restrict__ row_seq,
-                                  const int32_t* __restrict__ seq_slot,
-                                  const int32_t* __restrict__ seq_start,
-                                  const int32_t* __restrict__ seq_count, size_t total, int C) {
-  const size_t first = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
-  for (size_t idx = first; idx < total; idx += step) {
-    const size_t row = idx / C;
-    const int c = static_cast<int>(idx % C);
-    const int seq = row_seq[row];
-    if (seq < 0) continue;
-    const int start = seq_start[seq], count = seq_count[seq];
-    if (row_pos[row] != start + count - 1) continue;
-    float* tail = state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+                                  size_t tail_offset, const int32_t* __restrict__ seq_slot,
+                                  const int32_t* __restrict__ seq_count,
+                                  const int32_t* __restrict__ seq_row0, int C) {
+  const int seq = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int count = seq_count[seq];
+  if (count <= 0 || c >= C) return;          // padding of a fixed-size batch
+  const size_t row = static_cast<size_t>(seq_row0[seq]) + count - 1;     // the last row
+  float* tail = state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+  auto kept = [&](int i) {                    // what place i of the new tail holds
+    const int back = J - 2 - i;               // the input `back` positions before the last row
+    return back < count ? slice_sum(proj + (row - back) * WP + c, nsplit, split_stride)
+                        : tail[static_cast<size_t>(i + count) * C + c];
+  };
+  if (J - 1 <= kFewTaps) {
+    float keep[kFewTaps];
+#pragma unroll
+    for (int i = 0; i < kFewTaps; ++i) keep[i] = i < J - 1 ? kept(i) : 0.f;
+#pragma unroll
+    for (int i = 0; i < kFewTaps; ++i)
+      if (i < J - 1) tail[static_cast<size_t>(i) * C + c] = keep[i];
+  } else {
     float keep[kMaxTaps - 1];
-    for (int i = 0; i < J - 1; ++i) {
-      const int back = J - 2 - i;               // the input `back` positions before the last row
-      keep[i] = back < count ? slice_sum(proj + (row - back) * WP + c, nsplit, split_stride)
-                             : tail[static_cast<size_t>(i + count) * C + c];
-    }
+    for (int i = 0; i < J - 1; ++i) keep[i] = kept(i);
     for (int i = 0; i < J - 1; ++i) tail[static_cast<size_t>(i) * C + c] = keep[i];
   }
 }
@@ -196,28 +213,76 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
   }
   const float rate = expf(a_log[head]), shift = dt_bias[head];
 
-  for (int t0 = 0; t0 < count; t0 += TILE) {
-    const int nt = min(TILE, count - t0);
-    __syncthreads();                      // the last tile has been read
-    for (int idx = tid; idx < nt * DP; idx += kThreads) {
-      const int tt = idx / DP, i = idx % DP;
-      const float* src = conv + static_cast<size_t>(row0 + t0 + tt) * C + shared_head * D + i;
-      q_s[tt][i] = i < D ? src[0] : 0.f;
-      k_s[tt][i] = i < D ? src[QK] : 0.f;
+  // A tile's operands travel global memory -> registers -> LDS, and the registers are filled
+  // for tile t + 1 while tile t is walked, so the walk does not wait for memory.  Rows of q, k
+  // come as 16-byte pieces where the sizes allow (FAST), else element by element.
+  constexpr int QUADS = DP / 4;                          // 16-byte pieces of a padded q or k row
+  constexpr int NQ = (TILE * QUADS + kThreads - 1) / kThreads;   // pieces a thread moves per tile
+  constexpr int NV = (TILE * CB + kThreads - 1) / kThreads;      // values a thread moves per tile
+  const bool fast = D % 4 == 0 && C % 4 == 0;
+  float4 fq[NQ], fk[NQ];
+  float fv[NV], fb = 0.f, fa = 0.f;
+  auto fetch = [&](int t0, int nt) __attribute__((always_inline)) {
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+      const int idx = tid + n * kThreads, tt = idx / QUADS, i = (idx % QUADS) * 4;
+      fq[n] = fk[n] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (tt < nt && i < D) {
+        const float* src = conv + static_cast<size_t>(row0 + t0 + tt) * C + shared_head * D + i;
+        if (fast) {
+          fq[n] = *reinterpret_cast<const float4*>(src);
+          fk[n] = *reinterpret_cast<const float4*>(src + QK);
+        } else {
+          float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (i + e < D) {
+              a[e] = src[e];
+              b[e] = src[QK + e];
+            }
+          fq[n] = make_float4(a[0], a[1], a[2], a[3]);
+          fk[n] = make_float4(b[0], b[1], b[2], b[3]);
+        }
+      }
     }
-    for (int idx = tid; idx < nt * CB; idx += kThreads) {
-      const int tt = idx / CB, jj = idx % CB;
-      const int cg = blockIdx.z * CB + jj;
-      v_s[tt][jj] = cg < DV ? conv[static_cast<size_t>(row0 + t0 + tt) * C + 2 * QK + head * DV + cg]
-                            : 0.f;
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int idx = tid + n * kThreads, tt = idx / CB, cg = blockIdx.z * CB + idx % CB;
+      fv[n] = (tt < nt && cg < DV)
+                  ? conv[static_cast<size_t>(row0 + t0 + tt) * C + 2 * QK + head * DV + cg] : 0.f;
     }
     if (tid < nt) {
       const TI* src = proj + static_cast<size_t>(row0 + t0 + tid) * WP;
-      const float b = slice_sum(src + beta_col + head, nsplit, split_stride);
-      const float a = slice_sum(src + decay_col + head, nsplit, split_stride);
-      beta_s[tid] = 1.0f / (1.0f + expf(-b));
-      decay_s[tid] = expf(-rate * softplus_f32(a + shift));
+      fb = slice_sum(src + beta_col + head, nsplit, split_stride);
+      fa = slice_sum(src + decay_col + head, nsplit, split_stride);
     }
+  };
+  auto commit = [&](int nt) __attribute__((always_inline)) {
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+      const int idx = tid + n * kThreads, tt = idx / QUADS, i = (idx % QUADS) * 4;
+      if (tt < TILE) {
+        *reinterpret_cast<float4*>(&q_s[tt][i]) = fq[n];
+        *reinterpret_cast<float4*>(&k_s[tt][i]) = fk[n];
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int idx = tid + n * kThreads;
+      if (idx / CB < TILE) v_s[idx / CB][idx % CB] = fv[n];
+    }
+    if (tid < nt) {
+      beta_s[tid] = 1.0f / (1.0f + expf(-fb));
+      decay_s[tid] = expf(-rate * softplus_f32(fa + shift));
+    }
+  };
+
+  fetch(0, min(TILE, count));
+  for (int t0 = 0; t0 < count; t0 += TILE) {
+    const int nt = min(TILE, count - t0);
+    __syncthreads();                      // the last tile has been walked
+    commit(nt);
+    if (t0 + TILE < count) fetch(t0 + TILE, min(TILE, count - t0 - TILE));
     __syncthreads();
     {   // the factors that make q and k unit vectors: 8 threads a token
       const int tt = tid / 8, sub = tid % 8;
@@ -288,31 +353,31 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
   }
 }
 
-// One wave per (row, head): out = o / sqrt(mean(o^2) + eps) * w * silu(gate).
+// A block a row, its four waves over the heads: out = o / sqrt(mean(o^2) + eps) * w * silu(gate).
 template <typename TI, typename TO>
 __global__ void delta_out_kernel(const float* __restrict__ o_raw, const TI* __restrict__ proj,
                                  int nsplit, size_t split_stride, int WP, int gate_col,
                                  const float* __restrict__ norm_w, float eps,
                                  const int32_t* __restrict__ row_seq, TO* __restrict__ out,
-                                 long long items, int H, int DV) {
-  const long long item = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) / EI_WAVE;
-  const int lane = threadIdx.x % EI_WAVE;
-  if (item >= items) return;
-  const long long row = item / H;
-  const int head = static_cast<int>(item % H);
-  const size_t base = static_cast<size_t>(row) * H * DV + static_cast<size_t>(head) * DV;
-  if (row_seq[row] < 0) {                 // padding row: a defined input for the next product
-    for (int j = lane; j < DV; j += EI_WAVE) out[base + j] = ei::from_f32<TO>(0.f);
-    return;
-  }
-  float sq = 0.f;
-  for (int j = lane; j < DV; j += EI_WAVE) sq += o_raw[base + j] * o_raw[base + j];
-  sq = ei::wave_sum(sq);
-  const float inv = 1.0f / sqrtf(sq / static_cast<float>(DV) + eps);
-  const TI* gate = proj + static_cast<size_t>(row) * WP + gate_col + static_cast<size_t>(head) * DV;
-  for (int j = lane; j < DV; j += EI_WAVE) {
-    const float gt = slice_sum(gate + j, nsplit, split_stride);
-    out[base + j] = ei::from_f32<TO>((o_raw[base + j] * inv) * norm_w[j] * silu_f32(gt));
+                                 int H, int DV) {
+  const size_t row = blockIdx.x;
+  const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
+  const bool padding = row_seq[row] < 0;      // a defined input for the next product
+  for (int head = wave; head < H; head += kThreads / EI_WAVE) {
+    const size_t base = (row * H + head) * DV;
+    if (padding) {
+      for (int j = lane; j < DV; j += EI_WAVE) out[base + j] = ei::from_f32<TO>(0.f);
+      continue;
+    }
+    const TI* gate = proj + row * WP + gate_col + static_cast<size_t>(head) * DV;
+    float sq = 0.f;
+    for (int j = lane; j < DV; j += EI_WAVE) sq += o_raw[base + j] * o_raw[base + j];
+    sq = ei::wave_sum(sq);
+    const float inv = 1.0f / sqrtf(sq / static_cast<float>(DV) + eps);
+    for (int j = lane; j < DV; j += EI_WAVE) {
+      const float gt = slice_sum(gate + j, nsplit, split_stride);
+      out[base + j] = ei::from_f32<TO>((o_raw[base + j] * inv) * norm_w[j] * silu_f32(gt));
+    }
   }
 }
 
@@ -322,36 +387,33 @@ int lanes_a_column(int D) {
   return lanes;
 }
 
-unsigned grid_for(size_t total) {
-  size_t blocks = (total + kThreads - 1) / kThreads;
-  const size_t most = static_cast<size_t>(ei_compute_units()) * 32;
-  return static_cast<unsigned>(blocks > most ? most : blocks);
-}
-
 }  // namespace
 
 extern "C" int ei_delta_conv(const void* proj, int in_dtype, int nsplit, long long split_stride,
                              int WP, const float* conv_w, int J, const float* state,
                              long long state_stride, long long tail_offset, const int32_t* row_pos,
                              const int32_t* row_seq, const int32_t* seq_slot,
-                             const int32_t* seq_start, float* out, int N, int C,
+                             const int32_t* seq_start, float* out, int N, int C, int renew_tail,
                              hipStream_t stream) {
   EI_REQUIRE(proj && conv_w && state && row_pos && row_seq && seq_slot && seq_start && out,
              "delta_conv: null pointer");
+  EI_REQUIRE(!renew_tail || J <= kFewTaps, "delta_conv: the tails are renewed here for up to 8 taps");
+  float* renewed = renew_tail ? const_cast<float*>(state) : nullptr;
   EI_REQUIRE(N > 0 && C > 0 && C <= WP && nsplit >= 1, "delta_conv: sizes must be positive");
   EI_REQUIRE(J >= 1 && J <= kMaxTaps, "delta_conv: taps must lie between 1 and 32");
-  const size_t total = static_cast<size_t>(N) * C;
+  EI_REQUIRE((C + kThreads - 1) / kThreads <= 65535, "delta_conv: too many channels");
+  const dim3 grid(N, (C + kThreads - 1) / kThreads);
   const size_t ss = static_cast<size_t>(split_stride);
   if (in_dtype == EI_F32)
-    delta_conv_kernel<float><<<grid_for(total), kThreads, 0, stream>>>(
+    delta_conv_kernel<float><<<grid, kThreads, 0, stream>>>(
         static_cast<const float*>(proj), nsplit, ss, WP, conv_w, J, state,
         static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
-        seq_slot, seq_start, out, total, C);
+        seq_slot, seq_start, out, C, renewed);
   else if (in_dtype == EI_BF16)
-    delta_conv_kernel<bf16_t><<<grid_for(total), kThreads, 0, stream>>>(
+    delta_conv_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(
         static_cast<const bf16_t*>(proj), nsplit, ss, WP, conv_w, J, state,
         static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
-        seq_slot, seq_start, out, total, C);
+        seq_slot, seq_start, out, C, renewed);
   else
     EI_REQUIRE(false, "delta_conv: unknown dtype");
   EI_LAUNCH_CHECK();
@@ -359,25 +421,25 @@ extern "C" int ei_delta_conv(const void* proj, int in_dtype, int nsplit, long lo
 
 extern "C" int ei_delta_tail(const void* proj, int in_dtype, int nsplit, long long split_stride,
                              int WP, int J, float* state, long long state_stride,
-                             long long tail_offset, const int32_t* row_pos, const int32_t* row_seq,
-                             const int32_t* seq_slot, const int32_t* seq_start,
-                             const int32_t* seq_count, int N, int C, hipStream_t stream) {
-  EI_REQUIRE(proj && state && row_pos && row_seq && seq_slot && seq_start && seq_count,
-             "delta_tail: null pointer");
-  EI_REQUIRE(N > 0 && C > 0 && C <= WP && nsplit >= 1, "delta_tail: sizes must be positive");
+                             long long tail_offset, const int32_t* seq_slot,
+                             const int32_t* seq_count, const int32_t* seq_row0, int n_seqs, int C,
+                             hipStream_t stream) {
+  EI_REQUIRE(proj && state && seq_slot && seq_count && seq_row0, "delta_tail: null pointer");
+  EI_REQUIRE(n_seqs > 0 && C > 0 && C <= WP && nsplit >= 1, "delta_tail: sizes must be positive");
   EI_REQUIRE(J >= 2 && J <= kMaxTaps, "delta_tail: taps must lie between 2 and 32");
-  const size_t total = static_cast<size_t>(N) * C;
+  EI_REQUIRE((C + kThreads - 1) / kThreads <= 65535, "delta_tail: too many channels");
+  const dim3 grid(n_seqs, (C + kThreads - 1) / kThreads);
   const size_t ss = static_cast<size_t>(split_stride);
   if (in_dtype == EI_F32)
-    delta_tail_kernel<float><<<grid_for(total), kThreads, 0, stream>>>(
+    delta_tail_kernel<float><<<grid, kThreads, 0, stream>>>(
         static_cast<const float*>(proj), nsplit, ss, WP, J, state,
-        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
-        seq_slot, seq_start, seq_count, total, C);
+        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), seq_slot, seq_count,
+        seq_row0, C);
   else if (in_dtype == EI_BF16)
-    delta_tail_kernel<bf16_t><<<grid_for(total), kThreads, 0, stream>>>(
+    delta_tail_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(
         static_cast<const bf16_t*>(proj), nsplit, ss, WP, J, state,
-        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
-        seq_slot, seq_start, seq_count, total, C);
+        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), seq_slot, seq_count,
+        seq_row0, C);
   else
     EI_REQUIRE(false, "delta_tail: unknown dtype");
   EI_LAUNCH_CHECK();
@@ -435,14 +497,11 @@ extern "C" int ei_delta_out(const float* o_raw, const void* proj, int in_dtype, 
   EI_REQUIRE(N > 0 && H > 0 && DV > 0 && nsplit >= 1, "delta_out: sizes must be positive");
   EI_REQUIRE(gate_col >= 0 && gate_col + H * DV <= WP, "delta_out: gate columns outside the row");
   EI_REQUIRE(eps > 0.f, "delta_out: eps must be positive");
-  const long long items = static_cast<long long>(N) * H;
-  const long long blocks = (items * EI_WAVE + kThreads - 1) / kThreads;
-  EI_REQUIRE(blocks < (1ll << 31), "delta_out: too many rows");
   const size_t ss = static_cast<size_t>(split_stride);
 #define EI_DOUT(TI, TO)                                                                      \
-  delta_out_kernel<TI, TO><<<static_cast<unsigned>(blocks), kThreads, 0, stream>>>(          \
+  delta_out_kernel<TI, TO><<<N, kThreads, 0, stream>>>(                                      \
       o_raw, static_cast<const TI*>(proj), nsplit, ss, WP, gate_col, norm_w, eps, row_seq,   \
-      static_cast<TO*>(out), items, H, DV)
+      static_cast<TO*>(out), H, DV)
   if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_DOUT(float, float);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_DOUT(float, bf16_t);
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_DOUT(bf16_t, bf16_t);

@@ -42,7 +42,7 @@ _SIGNATURES = {
                                   c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                   c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p],
-        "ei_projection_norm_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
+        "ei_projection_norm_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p,
                                      c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_int, c_void_p],
@@ -50,10 +50,9 @@ _SIGNATURES = {
     "delta_rule": {
         "ei_delta_conv": [c_void_p, c_int, c_int, c_longlong, c_int, c_void_p, c_int, c_void_p,
                           c_longlong, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_void_p],
+                          c_int, c_int, c_int, c_void_p],
         "ei_delta_tail": [c_void_p, c_int, c_int, c_longlong, c_int, c_int, c_void_p, c_longlong,
-                          c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                          c_int, c_void_p],
+                          c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ei_delta_rule": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_int, c_int, c_int,
                           c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
@@ -443,14 +442,16 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
 
 def projection_norm_store(qkv, q_norm_w, k_norm_w, eps, row_pos, row_seq, page_table, q_out,
                           k_pages, v_pages, n_heads, n_kv_heads, head_dim, value_dim,
-                          write_cache=True) -> None:
+                          write_cache=True, bias=None) -> None:
     """One RMS norm over the whole query projection and one over the whole key projection
     (weights [heads * head_dim] and [kv heads * head_dim], or None for no norm), no rotation;
     queries to `q_out`, keys [*, kv heads, 64, head_dim] and values [*, kv heads, 64, value_dim]
-    to their cache pages."""
+    to their cache pages.  bias: float32 [q | k | v width], added to the projection first."""
     lib = library("rope_store")
     n = q_out.shape[0]
     width = n_heads * head_dim + n_kv_heads * (head_dim + value_dim)
+    if bias is not None and bias.numel() != width:
+        raise KernelError("projection_norm_store: the bias must be as wide as the projection")
     nsplit, stride = _splits(qkv, n, width, "qkv")
     if tuple(q_out.shape) != (n, n_heads * head_dim):
         raise KernelError("projection_norm_store: q_out has the wrong shape")
@@ -469,6 +470,7 @@ def projection_norm_store(qkv, q_norm_w, k_norm_w, eps, row_pos, row_seq, page_t
             raise KernelError("projection_norm_store: cache and q_out dtypes differ")
     status = lib.ei_projection_norm_store(
         _gpu(qkv, "qkv"), _code(qkv, "qkv"), nsplit, stride,
+        None if bias is None else _gpu(bias, "bias", torch.float32),
         None if q_norm_w is None else _gpu(q_norm_w, "q_norm", torch.float32),
         None if k_norm_w is None else _gpu(k_norm_w, "k_norm", torch.float32), float(eps),
         _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
@@ -692,11 +694,17 @@ def _delta_state(state, shape):
     return _gpu(state, "state", torch.float32)
 
 
+DELTA_FEW_TAPS = 8      # up to so many taps `delta_conv` can renew the tails itself
+
+
 def delta_conv(proj, conv_w, state, shape: DeltaShape, row_pos, row_seq, seq_slot, seq_start,
-               out) -> None:
+               out, renew_tail=False) -> None:
     """out [rows, channels] float32 = silu(causal convolution) of the q, k, v columns of
     `proj` ([rows, width] or float32 slices of it); conv_w float32 [channels, taps]; inputs
-    from before this step come from the sequences' tails in `state` [slots, state_floats]."""
+    from before this step come from the sequences' tails in `state` [slots, state_floats].
+    renew_tail: every sequence brings exactly one row (the caller vouches for it) and the
+    tails become the last taps - 1 inputs here, so `delta_tail` is not needed (at most
+    `DELTA_FEW_TAPS` taps)."""
     lib = library("delta_rule")
     rows = out.shape[0]
     if tuple(out.shape) != (rows, shape.channels) or tuple(conv_w.shape) != (shape.channels, shape.taps):
@@ -711,24 +719,26 @@ def delta_conv(proj, conv_w, state, shape: DeltaShape, row_pos, row_seq, seq_slo
                                _gpu(row_seq, "row_seq", torch.int32),
                                _gpu(seq_slot, "seq_slot", torch.int32),
                                _gpu(seq_start, "seq_start", torch.int32),
-                               _gpu(out, "out", torch.float32), rows, shape.channels, _stream())
+                               _gpu(out, "out", torch.float32), rows, shape.channels,
+                               int(bool(renew_tail)), _stream())
     _check(lib, status, "delta_conv")
 
 
-def delta_tail(proj, state, shape: DeltaShape, rows, row_pos, row_seq, seq_slot, seq_start,
-               seq_count) -> None:
-    """The sequences' tails in `state` become the last taps - 1 inputs after this step."""
+def delta_tail(proj, state, shape: DeltaShape, rows, seq_slot, seq_count, seq_row0) -> None:
+    """The sequences' tails in `state` become the last taps - 1 inputs after this step (of
+    `rows` packed rows; sequence s brings seq_count[s] of them from row seq_row0[s] on)."""
     if shape.taps < 2:
         return
     lib = library("delta_rule")
+    n_seqs = seq_count.numel()
+    if seq_slot.numel() < n_seqs or seq_row0.numel() < n_seqs:
+        raise KernelError("delta_tail: sequence metadata shorter than the sequences")
     pointer, code, nsplit, stride = _delta_proj(proj, rows, shape)
     status = lib.ei_delta_tail(pointer, code, nsplit, stride, shape.width, shape.taps,
                                _delta_state(state, shape), shape.state_floats, shape.tail_offset,
-                               _gpu(row_pos, "row_pos", torch.int32),
-                               _gpu(row_seq, "row_seq", torch.int32),
                                _gpu(seq_slot, "seq_slot", torch.int32),
-                               _gpu(seq_start, "seq_start", torch.int32),
-                               _gpu(seq_count, "seq_count", torch.int32), rows, shape.channels,
+                               _gpu(seq_count, "seq_count", torch.int32),
+                               _gpu(seq_row0, "seq_row0", torch.int32), n_seqs, shape.channels,
                                _stream())
     _check(lib, status, "delta_tail")
 

@@ -356,14 +356,15 @@ extern "C" int ei_qk_norm_rope_store(
 // head size may differ from the keys'.  One block a row; sums in float32, one rounding.
 namespace {
 
-template <typename TI, typename TO>
+template <typename TI, typename TO, bool VEC>
 __global__ void projection_norm_store_kernel(
-    const TI* __restrict__ qkv, int nsplit, size_t split_stride, const float* __restrict__ q_norm_w,
-    const float* __restrict__ k_norm_w, float eps, const int32_t* __restrict__ row_pos,
-    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
-    TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages, int nq, int nkv,
-    int D, int DV, int write_cache) {
-  extern __shared__ float row_values[];     // the row's q, k and v sums
+    const TI* __restrict__ qkv, int nsplit, size_t split_stride, const float* __restrict__ bias,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ page_table, int table_width, TO* __restrict__ q_out,
+    TO* __restrict__ k_pages, TO* __restrict__ v_pages, int nq, int nkv, int D, int DV,
+    int write_cache) {
+  extern __shared__ __attribute__((aligned(16))) float row_values[];     // the row's q, k and v sums
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const int seq = row_seq[row];
@@ -371,34 +372,84 @@ __global__ void projection_norm_store_kernel(
   const int QW = nq * D, KW = nkv * D, VW = nkv * DV, W = QW + KW + VW;
   const TI* src = qkv + static_cast<size_t>(row) * W;
   float q_sq = 0.f, k_sq = 0.f;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float x = 0.f;
-    for (int s0 = 0; s0 < nsplit; s0 += 8) {      // eight slices per trip to memory
-      float v[8];
+  if constexpr (VEC) {      // every width a multiple of 4: 16-byte pieces, 8 slices per trip
+    for (int i = threadIdx.x * 4; i < W; i += blockDim.x * 4) {
+      float x[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) ei::Vec4<float>::load(bias + i, x);
+      for (int s0 = 0; s0 < nsplit; s0 += 8) {
+        float v[8][4];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (s0 + u < nsplit) v[u] = ei::to_f32<TI>(src[(s0 + u) * split_stride + i]);
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) ei::Vec4<TI>::load(src + (s0 + u) * split_stride + i, v[u]);
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (s0 + u < nsplit) x += v[u];
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] += v[u][e];
+          }
+      }
+      ei::Vec4<float>::store(row_values + i, x);
+      const float sq = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+      if (i < QW) q_sq += sq;
+      else if (i < QW + KW) k_sq += sq;
     }
-    row_values[i] = x;
-    if (i < QW) q_sq += x * x;
-    else if (i < QW + KW) k_sq += x * x;
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      float x = bias ? bias[i] : 0.f;
+      for (int s0 = 0; s0 < nsplit; s0 += 8) {      // eight slices per trip to memory
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) v[u] = ei::to_f32<TI>(src[(s0 + u) * split_stride + i]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) x += v[u];
+      }
+      row_values[i] = x;
+      if (i < QW) q_sq += x * x;
+      else if (i < QW + KW) k_sq += x * x;
+    }
   }
   const float q_total = ei::block_sum(q_sq, scratch);
   const float k_total = ei::block_sum(k_sq, scratch);
   const float q_inv = q_norm_w ? 1.0f / sqrtf(q_total / static_cast<float>(QW) + eps) : 1.f;
   const float k_inv = k_norm_w ? 1.0f / sqrtf(k_total / static_cast<float>(KW) + eps) : 1.f;
+  const int pos = row_pos[row];
+  const int phys = write_cache ? page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE] : -1;
+  const int in_page = pos % EI_PAGE;
+  if constexpr (VEC) {
+    for (int i = threadIdx.x * 4; i < W; i += blockDim.x * 4) {
+      float x[4], w[4] = {1.f, 1.f, 1.f, 1.f};
+      ei::Vec4<float>::load(row_values + i, x);
+      if (i < QW) {
+        if (q_norm_w) {
+          ei::Vec4<float>::load(q_norm_w + i, w);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) x[e] = (x[e] * q_inv) * w[e];
+        }
+        ei::Vec4<TO>::store(q_out + static_cast<size_t>(row) * QW + i, x);
+      } else if (phys >= 0 && i < QW + KW) {
+        const int at = i - QW, head = at / D, d = at % D;
+        if (k_norm_w) {
+          ei::Vec4<float>::load(k_norm_w + at, w);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) x[e] = (x[e] * k_inv) * w[e];
+        }
+        ei::Vec4<TO>::store(
+            k_pages + ((static_cast<size_t>(phys) * nkv + head) * EI_PAGE + in_page) * D + d, x);
+      } else if (phys >= 0) {
+        const int at = i - QW - KW, head = at / DV, d = at % DV;
+        ei::Vec4<TO>::store(
+            v_pages + ((static_cast<size_t>(phys) * nkv + head) * EI_PAGE + in_page) * DV + d, x);
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < QW; i += blockDim.x) {
     const float y = q_norm_w ? (row_values[i] * q_inv) * q_norm_w[i] : row_values[i];
     q_out[static_cast<size_t>(row) * QW + i] = ei::from_f32<TO>(y);
   }
-  if (!write_cache) return;
-  const int pos = row_pos[row];
-  const int phys = page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE];
   if (phys < 0) return;
-  const int in_page = pos % EI_PAGE;
   for (int i = threadIdx.x; i < KW; i += blockDim.x) {
     const int head = i / D, d = i % D;
     const float x = row_values[QW + i];
@@ -417,9 +468,11 @@ __global__ void projection_norm_store_kernel(
 
 // qkv: [nsplit][N, nq * D + nkv * D + nkv * DV] of in_dtype; q_out: [N, nq * D]; key pages
 // [n_pages, nkv, 64, D], value pages [n_pages, nkv, 64, DV] of out_dtype; q_norm_w [nq * D] and
-// k_norm_w [nkv * D] float32, or both null (no norm).
+// k_norm_w [nkv * D] float32, or both null (no norm); bias: float32 [row width] added to the
+// sums, or null.
 extern "C" int ei_projection_norm_store(
-    const void* qkv, int in_dtype, int nsplit, long long split_stride, const float* q_norm_w,
+    const void* qkv, int in_dtype, int nsplit, long long split_stride, const float* bias,
+    const float* q_norm_w,
     const float* k_norm_w, float eps, const int32_t* row_pos, const int32_t* row_seq,
     const int32_t* page_table, int table_width, void* q_out, void* k_pages, void* v_pages,
     int out_dtype, int N, int nq, int nkv, int D, int DV, int write_cache, hipStream_t stream) {
@@ -436,21 +489,32 @@ extern "C" int ei_projection_norm_store(
   const size_t lds = static_cast<size_t>(width) * sizeof(float);
   const int threads = width >= 2048 ? 512 : 256;
   const size_t ss = static_cast<size_t>(split_stride);
-#define EI_PNS(TI, TO)                                                                          \
+  const bool aligned = (reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(q_out) |
+                        reinterpret_cast<uintptr_t>(k_pages) | reinterpret_cast<uintptr_t>(v_pages) |
+                        reinterpret_cast<uintptr_t>(q_norm_w) | reinterpret_cast<uintptr_t>(k_norm_w) |
+                        reinterpret_cast<uintptr_t>(bias)) % 16 == 0;
+  const bool vec = D % 4 == 0 && DV % 4 == 0 && ss % 4 == 0 && aligned;
+#define EI_PNS_V(TI, TO, VV)                                                                    \
   do {                                                                                          \
     if (lds > 64 * 1024)                                                                        \
       (void)hipFuncSetAttribute(                                                                \
-          reinterpret_cast<const void*>(&projection_norm_store_kernel<TI, TO>),                 \
+          reinterpret_cast<const void*>(&projection_norm_store_kernel<TI, TO, VV>),             \
           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));                   \
-    projection_norm_store_kernel<TI, TO><<<N, threads, lds, stream>>>(                          \
-        static_cast<const TI*>(qkv), nsplit, ss, q_norm_w, k_norm_w, eps, row_pos, row_seq,     \
-        page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),            \
+    projection_norm_store_kernel<TI, TO, VV><<<N, threads, lds, stream>>>(                      \
+        static_cast<const TI*>(qkv), nsplit, ss, bias, q_norm_w, k_norm_w, eps, row_pos,        \
+        row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),   \
         static_cast<TO*>(v_pages), nq, nkv, D, DV, write_cache);                                \
+  } while (0)
+#define EI_PNS(TI, TO)                 \
+  do {                                 \
+    if (vec) EI_PNS_V(TI, TO, true);   \
+    else EI_PNS_V(TI, TO, false);      \
   } while (0)
   if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_PNS(float, float);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_PNS(float, bf16_t);
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_PNS(bf16_t, bf16_t);
   else EI_REQUIRE(false, "projection_norm_store: unsupported dtype combination");
 #undef EI_PNS
+#undef EI_PNS_V
   EI_LAUNCH_CHECK();
 }

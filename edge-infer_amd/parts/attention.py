@@ -306,7 +306,9 @@ class Attention:
         meta = ctx.meta
         group_index, k_pages, v_pages = ctx.cache.kv(entry.cache)
         page_table = meta.page_table(group_index)
-        qkv = self.qkv.forward(ctx, x, "attn.qkv")
+        # (the kernel that norms and stores the whole projection adds its bias as well)
+        qkv, bias = (self.qkv.forward(ctx, x, "attn.qkv", bias_later=True) if self.whole_store
+                     else (self.qkv.forward(ctx, x, "attn.qkv"), None))
         if (ctx.decode and self.matrix_cores and FUSED_DECODE and qkv.dim() == 3
                 and qkv.dtype == torch.float32 and not self.whole_store and not self.has_extras):
             # the decode kernel norms, rotates and stores for its rows itself: one launch less
@@ -317,7 +319,7 @@ class Attention:
             lib.projection_norm_store(
                 qkv, self.q_norm, self.k_norm, spec.qk_norm_eps, meta.row_pos, meta.row_seq,
                 page_table, q, k_pages, v_pages, spec.n_heads, spec.n_kv_heads, spec.head_dim,
-                spec.v_dim, write_cache=entry.writes_cache)
+                spec.v_dim, write_cache=entry.writes_cache, bias=bias)
         else:
             q = ctx.buffer("attn.q", (n, spec.q_width))
             lib.qk_norm_rope_store(

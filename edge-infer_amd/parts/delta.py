@@ -105,11 +105,12 @@ class GatedDelta:
         state = ctx.cache.state(entry.cache)                 # [slots + 1, state_floats]
         proj = self.proj.forward(ctx, x, "delta.proj")
         conv = ctx.buffer("delta.conv", (n, shape.channels), torch.float32)
+        # a decode step (one row a sequence) renews the convolution's tails in the same kernel
+        renew = ctx.decode and entry.writes_cache and shape.taps <= lib.DELTA_FEW_TAPS
         lib.delta_conv(proj, self.conv_w, state, shape, meta.row_pos, meta.row_seq,
-                       meta.seq_slot, meta.seq_start, conv)
-        if entry.writes_cache:
-            lib.delta_tail(proj, state, shape, n, meta.row_pos, meta.row_seq, meta.seq_slot,
-                           meta.seq_start, meta.seq_count)
+                       meta.seq_slot, meta.seq_start, conv, renew_tail=renew)
+        if entry.writes_cache and not renew:
+            lib.delta_tail(proj, state, shape, n, meta.seq_slot, meta.seq_count, meta.seq_row0)
         o_raw = ctx.buffer("delta.o_raw", (n, shape.v_width), torch.float32)
         lib.delta_rule(conv, proj, self.decay_log_rate, self.decay_bias, state, shape,
                        meta.seq_slot, meta.seq_count, meta.seq_row0, o_raw, self.q_scale,

@@ -76,28 +76,34 @@ class Linear:
         else:
             lib.gemm_bf16_skinny(x, self.weight, out)
 
-    def forward(self, ctx, x: torch.Tensor, out_name: str) -> torch.Tensor:
+    def forward(self, ctx, x: torch.Tensor, out_name: str, bias_later: bool = False):
         """x [N, in] of the step's storage type -> [N, out] in the storage type, or float32
         partial sums [slices, N, out] when the few-rows kernel ran; the result lives in the
-        workspace buffer `out_name`."""
+        workspace buffer `out_name`.  bias_later: the caller's next kernel adds the bias itself
+        where that saves a launch; the call then returns (result, float32 bias still to be
+        added or None)."""
         rows = x.shape[0]
+        own_launch = self.dtype == torch.float32 or lib.skinny_gemm_ok(rows, self.in_features)
+        leave = bias_later and self.bias is not None and own_launch
+        bias = None if leave else self.bias
         if self.dtype == torch.float32:
             out = ctx.buffer(out_name, (rows, self.out_features), torch.float32)
             lib.gemm_f32(x, self.weight, out)
-            if self.bias is not None:
+            if bias is not None:
                 lib.bias_rows(self.bias_f32, out, accumulate=True)
-            return out
-        if lib.skinny_gemm_ok(rows, self.in_features):
+        elif lib.skinny_gemm_ok(rows, self.in_features):
             splits = lib.skinny_gemm_splits(rows, self.out_features, self.in_features)
-            extra = 0 if self.bias is None else 1
+            extra = 0 if bias is None else 1
             out = ctx.buffer(out_name + ".f32", (splits + extra, rows, self.out_features),
                              torch.float32)
             self._few_rows(x, out[:splits])
             if extra:
                 lib.bias_rows(self.bias_f32, out[splits], accumulate=False)
-            return out
-        out = ctx.buffer(out_name, (rows, self.out_features), torch.bfloat16)
-        self._library(x, out)
+        else:
+            out = ctx.buffer(out_name, (rows, self.out_features), torch.bfloat16)
+            self._library(x, out)
+        if bias_later:
+            return out, (self.bias_f32 if leave else None)
         return out
 
     def _library(self, x: torch.Tensor, out: torch.Tensor) -> None:
