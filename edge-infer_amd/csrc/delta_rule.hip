@@ -353,7 +353,7 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
   }
 }
 
-// A block a row, its four waves over the heads: out = o / sqrt(mean(o^2) + eps) * w * silu(gate).
+// A wave a (row, head), four heads a block: out = o / sqrt(mean(o^2) + eps) * w * silu(gate).
 template <typename TI, typename TO>
 __global__ void delta_out_kernel(const float* __restrict__ o_raw, const TI* __restrict__ proj,
                                  int nsplit, size_t split_stride, int WP, int gate_col,
@@ -363,11 +363,12 @@ __global__ void delta_out_kernel(const float* __restrict__ o_raw, const TI* __re
   const size_t row = blockIdx.x;
   const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
   const bool padding = row_seq[row] < 0;      // a defined input for the next product
-  for (int head = wave; head < H; head += kThreads / EI_WAVE) {
+  const int head = blockIdx.y * (kThreads / EI_WAVE) + wave;
+  if (head < H) {
     const size_t base = (row * H + head) * DV;
     if (padding) {
       for (int j = lane; j < DV; j += EI_WAVE) out[base + j] = ei::from_f32<TO>(0.f);
-      continue;
+      return;
     }
     const TI* gate = proj + row * WP + gate_col + static_cast<size_t>(head) * DV;
     float sq = 0.f;
@@ -497,9 +498,10 @@ extern "C" int ei_delta_out(const float* o_raw, const void* proj, int in_dtype, 
   EI_REQUIRE(N > 0 && H > 0 && DV > 0 && nsplit >= 1, "delta_out: sizes must be positive");
   EI_REQUIRE(gate_col >= 0 && gate_col + H * DV <= WP, "delta_out: gate columns outside the row");
   EI_REQUIRE(eps > 0.f, "delta_out: eps must be positive");
+  EI_REQUIRE((H + 3) / 4 <= 65535, "delta_out: too many heads");
   const size_t ss = static_cast<size_t>(split_stride);
 #define EI_DOUT(TI, TO)                                                                      \
-  delta_out_kernel<TI, TO><<<N, kThreads, 0, stream>>>(                                      \
+  delta_out_kernel<TI, TO><<<dim3(N, (H + 3) / 4), kThreads, 0, stream>>>(                   \
       o_raw, static_cast<const TI*>(proj), nsplit, ss, WP, gate_col, norm_w, eps, row_seq,   \
       static_cast<TO*>(out), H, DV)
   if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_DOUT(float, float);

@@ -38,8 +38,8 @@ CONFIG_B = {"architecture": "Tirurax", "vocab": 97, "width": 96, "norm": {"eps":
                        delta(1, 1, 160, 12, 1, 64), attention(8, 2, 16, 16, 0.25, 7, 40)]}
 # head sizes 64 and 128 with values as wide as keys: what the matrix-core attention kernels take
 CONFIG_C = {"architecture": "Tirurax", "vocab": 150, "width": 128, "norm": {"eps": 1e-6},
-            "layers": [attention(4, 2, 64, 64, 0.15, 48, 160), delta(2, 2, 32, 64, 4, 96),
-                       attention(2, 1, 128, 128, 0.1, 200, None),
+            "layers": [attention(6, 2, 64, 64, 0.15, 48, 160), delta(2, 2, 32, 64, 4, 96),
+                       attention(3, 3, 128, 128, 0.1, 200, None),
                        attention(8, 2, 64, 64, 0.125, None, 64)]}
 CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
 
