@@ -356,6 +356,92 @@ extern "C" int ei_qk_norm_rope_store(
 // head size may differ from the keys'.  One block a row; sums in float32, one rounding.
 namespace {
 
+// The same for rows of at most 4 x 256 16-byte pieces whose widths are all multiples of 4: a
+// thread keeps its pieces in registers between the sums of squares and the stores, and the two
+// sums cross the block together.
+template <typename TI, typename TO, int CH>
+__global__ void __launch_bounds__(256)
+projection_norm_store_reg_kernel(
+    const TI* __restrict__ qkv, int nsplit, size_t split_stride, const float* __restrict__ bias,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ page_table, int table_width, TO* __restrict__ q_out,
+    TO* __restrict__ k_pages, TO* __restrict__ v_pages, int nq, int nkv, int D, int DV,
+    int write_cache) {
+  __shared__ float sums[2][4];
+  const int row = blockIdx.x;
+  const int seq = row_seq[row];
+  if (seq < 0) return;                      // padding row of a fixed-size batch
+  const int QW = nq * D, KW = nkv * D, VW = nkv * DV, W = QW + KW + VW;
+  const TI* src = qkv + static_cast<size_t>(row) * W;
+  float x[CH][4];
+  float q_sq = 0.f, k_sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (threadIdx.x + c * 256) * 4;
+    x[c][0] = x[c][1] = x[c][2] = x[c][3] = 0.f;
+    if (i < W) {
+      if (bias) ei::Vec4<float>::load(bias + i, x[c]);
+      for (int s0 = 0; s0 < nsplit; s0 += 8) {
+        float v[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) ei::Vec4<TI>::load(src + (s0 + u) * split_stride + i, v[u]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[c][e] += v[u][e];
+          }
+      }
+      const float sq = x[c][0] * x[c][0] + x[c][1] * x[c][1] + x[c][2] * x[c][2] + x[c][3] * x[c][3];
+      if (i < QW) q_sq += sq;
+      else if (i < QW + KW) k_sq += sq;
+    }
+  }
+  q_sq = ei::wave_sum(q_sq);
+  k_sq = ei::wave_sum(k_sq);
+  if (threadIdx.x % EI_WAVE == 0) {
+    sums[0][threadIdx.x / EI_WAVE] = q_sq;
+    sums[1][threadIdx.x / EI_WAVE] = k_sq;
+  }
+  __syncthreads();
+  const float q_total = sums[0][0] + sums[0][1] + sums[0][2] + sums[0][3];
+  const float k_total = sums[1][0] + sums[1][1] + sums[1][2] + sums[1][3];
+  const float q_inv = q_norm_w ? 1.0f / sqrtf(q_total / static_cast<float>(QW) + eps) : 1.f;
+  const float k_inv = k_norm_w ? 1.0f / sqrtf(k_total / static_cast<float>(KW) + eps) : 1.f;
+  const int pos = row_pos[row];
+  const int phys = write_cache ? page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE] : -1;
+  const int in_page = pos % EI_PAGE;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (threadIdx.x + c * 256) * 4;
+    if (i >= W) continue;
+    float w[4];
+    if (i < QW) {
+      if (q_norm_w) {
+        ei::Vec4<float>::load(q_norm_w + i, w);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[c][e] = (x[c][e] * q_inv) * w[e];
+      }
+      ei::Vec4<TO>::store(q_out + static_cast<size_t>(row) * QW + i, x[c]);
+    } else if (phys >= 0 && i < QW + KW) {
+      const int at = i - QW, head = at / D, d = at % D;
+      if (k_norm_w) {
+        ei::Vec4<float>::load(k_norm_w + at, w);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[c][e] = (x[c][e] * k_inv) * w[e];
+      }
+      ei::Vec4<TO>::store(
+          k_pages + ((static_cast<size_t>(phys) * nkv + head) * EI_PAGE + in_page) * D + d, x[c]);
+    } else if (phys >= 0) {
+      const int at = i - QW - KW, head = at / DV, d = at % DV;
+      ei::Vec4<TO>::store(
+          v_pages + ((static_cast<size_t>(phys) * nkv + head) * EI_PAGE + in_page) * DV + d, x[c]);
+    }
+  }
+}
+
 template <typename TI, typename TO, bool VEC>
 __global__ void projection_norm_store_kernel(
     const TI* __restrict__ qkv, int nsplit, size_t split_stride, const float* __restrict__ bias,
@@ -505,16 +591,25 @@ extern "C" int ei_projection_norm_store(
         row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),   \
         static_cast<TO*>(v_pages), nq, nkv, D, DV, write_cache);                                \
   } while (0)
-#define EI_PNS(TI, TO)                 \
-  do {                                 \
-    if (vec) EI_PNS_V(TI, TO, true);   \
-    else EI_PNS_V(TI, TO, false);      \
+#define EI_PNS_R(TI, TO, CC)                                                                    \
+  projection_norm_store_reg_kernel<TI, TO, CC><<<N, 256, 0, stream>>>(                          \
+      static_cast<const TI*>(qkv), nsplit, ss, bias, q_norm_w, k_norm_w, eps, row_pos, row_seq, \
+      page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),              \
+      static_cast<TO*>(v_pages), nq, nkv, D, DV, write_cache)
+#define EI_PNS(TI, TO)                                   \
+  do {                                                   \
+    if (vec && width <= 1024) EI_PNS_R(TI, TO, 1);       \
+    else if (vec && width <= 2048) EI_PNS_R(TI, TO, 2);  \
+    else if (vec && width <= 4096) EI_PNS_R(TI, TO, 4);  \
+    else if (vec) EI_PNS_V(TI, TO, true);                \
+    else EI_PNS_V(TI, TO, false);                        \
   } while (0)
   if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_PNS(float, float);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_PNS(float, bf16_t);
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_PNS(bf16_t, bf16_t);
   else EI_REQUIRE(false, "projection_norm_store: unsupported dtype combination");
 #undef EI_PNS
+#undef EI_PNS_R
 #undef EI_PNS_V
   EI_LAUNCH_CHECK();
 }
