@@ -27,7 +27,6 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kTile = 32;        // most tokens of a sequence that delta_rule stages in LDS at a time
-constexpr int kOwn = 8;          // rows of a column of S that one thread owns
 constexpr int kMaxTaps = 32;
 constexpr int kFewTaps = 8;      // up to so many taps a thread keeps a channel's inputs in registers
 
@@ -155,8 +154,14 @@ __device__ __forceinline__ float group_sum(float v) {
 }
 
 // conv: [N, C] = q [G * D] | k [G * D] | v [H * DV] after convolution and silu.  The block
-// (sequence, head, column block) walks the sequence's rows of this step in order.
-template <typename TI, int L>
+// (sequence, head, column block) walks the sequence's rows of this step in order.  A thread owns
+// OWN rows of one column of S, L neighbouring lanes share the column.  Per token, with S the
+// state before the token, g its decay, k, q the unit key and the scaled unit query:
+//   seen = g (S^T k)[col];  u = beta (v[col] - seen);  o[col] = g (S^T q)[col] + u (k . q);
+//   S[., col] <- g S[., col] + k u
+// (o = (g S + k u^T)^T q written out: both dot products are taken from the old S, so their
+// sums over the lanes run side by side and the update is off the read-out's path).
+template <typename TI, int L, int OWN>
 __global__ void __launch_bounds__(kThreads)
 delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ proj, int nsplit,
                   size_t split_stride, int WP, int beta_col, int decay_col,
@@ -165,15 +170,17 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
                   const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ seq_count,
                   const int32_t* __restrict__ seq_row0, float* __restrict__ o_raw, int H, int G,
                   int D, int DV, float q_scale, float unit_eps) {
-  constexpr int DP = L * kOwn;            // D rounded up to what the lanes of a column hold
+  constexpr int DP = L * OWN;             // D rounded up to what the lanes of a column hold
   constexpr int CB = kThreads / L;        // columns of S a block holds
-  constexpr int TILE = L >= 32 ? kTile / 2 : kTile;   // (the widest keys: half, to fit 64 KB)
+  constexpr int TILE = DP >= 256 ? kTile / 2 : kTile;   // (the widest keys: half, to fit 64 KB)
+  constexpr int PIECES = OWN / 4;         // 16-byte pieces of a thread's rows
   __shared__ __attribute__((aligned(16))) float q_s[TILE][DP];
   __shared__ __attribute__((aligned(16))) float k_s[TILE][DP];
   __shared__ float v_s[TILE][CB];
-  // per token: decay g, the factor that makes k a unit vector, beta times that factor, and
-  // the factor of q (unit vector times q_scale)
+  // per token: decay g, the factor kf that makes k a unit vector, beta kf, the factor qf of q
+  // (unit vector times q_scale); and qf (k . q) of the raw vectors
   __shared__ __attribute__((aligned(16))) float4 coef_s[TILE];
+  __shared__ float kq_s[TILE];
   __shared__ float beta_s[TILE], decay_s[TILE];
 
   const int seq = blockIdx.x;
@@ -185,29 +192,27 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
   const int col_in_block = tid / L, part = tid % L;
   const int col = blockIdx.z * CB + col_in_block;
   const bool col_ok = col < DV;
-  const int i0 = part * kOwn;
+  const int i0 = part * OWN;
   const int QK = G * D, VW = H * DV;
 
   float* mine = state + static_cast<size_t>(seq_slot[seq]) * state_stride +
                 (static_cast<size_t>(head) * DV + (col_ok ? col : 0)) * D + i0;
   // (D a multiple of 4: the rows a thread owns are whole 16-byte pieces, inside S or outside)
   const bool wide = D % 4 == 0;
-  float s[kOwn];
+  float s[OWN];
 #pragma unroll
-  for (int m = 0; m < kOwn; ++m) s[m] = 0.f;
+  for (int m = 0; m < OWN; ++m) s[m] = 0.f;
   if (col_ok) {
     if (wide) {
-      if (i0 < D) {
-        const float4 a = *reinterpret_cast<const float4*>(mine);
-        s[0] = a.x; s[1] = a.y; s[2] = a.z; s[3] = a.w;
-      }
-      if (i0 + 4 < D) {
-        const float4 a = *reinterpret_cast<const float4*>(mine + 4);
-        s[4] = a.x; s[5] = a.y; s[6] = a.z; s[7] = a.w;
-      }
+#pragma unroll
+      for (int pc = 0; pc < PIECES; ++pc)
+        if (i0 + 4 * pc < D) {
+          const float4 a = *reinterpret_cast<const float4*>(mine + 4 * pc);
+          s[4 * pc] = a.x; s[4 * pc + 1] = a.y; s[4 * pc + 2] = a.z; s[4 * pc + 3] = a.w;
+        }
     } else {
 #pragma unroll
-      for (int m = 0; m < kOwn; ++m)
+      for (int m = 0; m < OWN; ++m)
         if (i0 + m < D) s[m] = mine[m];
     }
   }
@@ -284,70 +289,78 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
     commit(nt);
     if (t0 + TILE < count) fetch(t0 + TILE, min(TILE, count - t0 - TILE));
     __syncthreads();
-    {   // the factors that make q and k unit vectors: 8 threads a token
+    {   // the factors that make q and k unit vectors, and k . q: 8 threads a token
       const int tt = tid / 8, sub = tid % 8;
-      float q_sq = 0.f, k_sq = 0.f;
+      float q_sq = 0.f, k_sq = 0.f, kq = 0.f;
       if (tt < nt)
         for (int i = sub; i < D; i += 8) {
           q_sq += q_s[tt][i] * q_s[tt][i];
           k_sq += k_s[tt][i] * k_s[tt][i];
+          kq += k_s[tt][i] * q_s[tt][i];
         }
       q_sq = group_sum<8>(q_sq);
       k_sq = group_sum<8>(k_sq);
+      kq = group_sum<8>(kq);
       if (tt < nt && sub == 0) {
-        const float kf = 1.0f / sqrtf(k_sq + unit_eps);
-        coef_s[tt] = make_float4(decay_s[tt], kf, beta_s[tt] * kf, q_scale / sqrtf(q_sq + unit_eps));
+        const float kf = 1.0f / sqrtf(k_sq + unit_eps), qf = q_scale / sqrtf(q_sq + unit_eps);
+        coef_s[tt] = make_float4(decay_s[tt], kf, beta_s[tt] * kf, qf);
+        kq_s[tt] = kq * qf;
       }
     }
     __syncthreads();
     // the walk: what token tt + 1 needs is read from LDS while token tt is computed
-    float4 ka = *reinterpret_cast<const float4*>(&k_s[0][i0]);
-    float4 kb = *reinterpret_cast<const float4*>(&k_s[0][i0 + 4]);
-    float4 qa = *reinterpret_cast<const float4*>(&q_s[0][i0]);
-    float4 qb = *reinterpret_cast<const float4*>(&q_s[0][i0 + 4]);
+    float4 kn[PIECES], qn[PIECES];
+#pragma unroll
+    for (int pc = 0; pc < PIECES; ++pc) {
+      kn[pc] = *reinterpret_cast<const float4*>(&k_s[0][i0 + 4 * pc]);
+      qn[pc] = *reinterpret_cast<const float4*>(&q_s[0][i0 + 4 * pc]);
+    }
     float4 cf = coef_s[0];
-    float vv = v_s[0][col_in_block];
+    float vv = v_s[0][col_in_block], kqv = kq_s[0];
     for (int tt = 0; tt < nt; ++tt) {
-      const float kv[kOwn] = {ka.x, ka.y, ka.z, ka.w, kb.x, kb.y, kb.z, kb.w};
-      const float qv[kOwn] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
-      const float g = cf.x, kf = cf.y, bk = cf.z, qf = cf.w, v_now = vv;
+      float kv[OWN], qv[OWN];
+#pragma unroll
+      for (int pc = 0; pc < PIECES; ++pc) {
+        kv[4 * pc] = kn[pc].x; kv[4 * pc + 1] = kn[pc].y; kv[4 * pc + 2] = kn[pc].z; kv[4 * pc + 3] = kn[pc].w;
+        qv[4 * pc] = qn[pc].x; qv[4 * pc + 1] = qn[pc].y; qv[4 * pc + 2] = qn[pc].z; qv[4 * pc + 3] = qn[pc].w;
+      }
+      const float g = cf.x, kf = cf.y, bk = cf.z, qf = cf.w, v_now = vv, kq_now = kqv;
       const int nx = tt + 1 < nt ? tt + 1 : tt;
-      ka = *reinterpret_cast<const float4*>(&k_s[nx][i0]);
-      kb = *reinterpret_cast<const float4*>(&k_s[nx][i0 + 4]);
-      qa = *reinterpret_cast<const float4*>(&q_s[nx][i0]);
-      qb = *reinterpret_cast<const float4*>(&q_s[nx][i0 + 4]);
+#pragma unroll
+      for (int pc = 0; pc < PIECES; ++pc) {
+        kn[pc] = *reinterpret_cast<const float4*>(&k_s[nx][i0 + 4 * pc]);
+        qn[pc] = *reinterpret_cast<const float4*>(&q_s[nx][i0 + 4 * pc]);
+      }
       cf = coef_s[nx];
       vv = v_s[nx][col_in_block];
-      float seen0 = 0.f, seen1 = 0.f;
+      kqv = kq_s[nx];
+      float seen0 = 0.f, seen1 = 0.f, read0 = 0.f, read1 = 0.f;
 #pragma unroll
-      for (int m = 0; m < kOwn; m += 2) {
-        s[m] *= g;
-        s[m + 1] *= g;
+      for (int m = 0; m < OWN; m += 2) {
         seen0 = fmaf(s[m], kv[m], seen0);
         seen1 = fmaf(s[m + 1], kv[m + 1], seen1);
+        read0 = fmaf(s[m], qv[m], read0);
+        read1 = fmaf(s[m + 1], qv[m + 1], read1);
       }
-      const float seen = group_sum<L>(seen0 + seen1) * kf;       // (S^T k)[col], k a unit vector
-      const float u = bk * (v_now - seen);                       // beta (v - S^T k), times k's factor
-      float o0 = 0.f, o1 = 0.f;
+      const float seen = group_sum<L>(seen0 + seen1) * (g * kf);    // g (S^T k)[col], k a unit vector
+      const float read = group_sum<L>(read0 + read1) * (g * qf);    // g (S^T q)[col]
+      const float u = bk * (v_now - seen);                          // beta (v - seen), times k's factor
 #pragma unroll
-      for (int m = 0; m < kOwn; m += 2) {
-        s[m] = fmaf(kv[m], u, s[m]);
-        s[m + 1] = fmaf(kv[m + 1], u, s[m + 1]);
-        o0 = fmaf(s[m], qv[m], o0);
-        o1 = fmaf(s[m + 1], qv[m + 1], o1);
-      }
-      const float o = group_sum<L>(o0 + o1) * qf;
+      for (int m = 0; m < OWN; ++m) s[m] = fmaf(s[m], g, kv[m] * u);
       if (part == 0 && col_ok)
-        o_raw[static_cast<size_t>(row0 + t0 + tt) * VW + head * DV + col] = o;
+        o_raw[static_cast<size_t>(row0 + t0 + tt) * VW + head * DV + col] = fmaf(u, kq_now, read);
     }
   }
   if (col_ok) {
     if (wide) {
-      if (i0 < D) *reinterpret_cast<float4*>(mine) = make_float4(s[0], s[1], s[2], s[3]);
-      if (i0 + 4 < D) *reinterpret_cast<float4*>(mine + 4) = make_float4(s[4], s[5], s[6], s[7]);
+#pragma unroll
+      for (int pc = 0; pc < PIECES; ++pc)
+        if (i0 + 4 * pc < D)
+          *reinterpret_cast<float4*>(mine + 4 * pc) =
+              make_float4(s[4 * pc], s[4 * pc + 1], s[4 * pc + 2], s[4 * pc + 3]);
     } else {
 #pragma unroll
-      for (int m = 0; m < kOwn; ++m)
+      for (int m = 0; m < OWN; ++m)
         if (i0 + m < D) mine[m] = s[m];
     }
   }
@@ -382,9 +395,9 @@ __global__ void delta_out_kernel(const float* __restrict__ o_raw, const TI* __re
   }
 }
 
-int lanes_a_column(int D) {
+int lanes_a_column(int D, int own) {
   int lanes = 1;
-  while (lanes * kOwn < D) lanes *= 2;
+  while (lanes * own < D) lanes *= 2;
   return lanes;
 }
 
@@ -462,29 +475,53 @@ extern "C" int ei_delta_rule(const float* conv, const void* proj, int in_dtype, 
   EI_REQUIRE(D >= 1 && D <= 256, "delta_rule: the key size must lie between 1 and 256");
   EI_REQUIRE(beta_col >= 0 && decay_col >= 0 && beta_col + H <= WP && decay_col + H <= WP,
              "delta_rule: projection columns outside the row");
-  const int L = lanes_a_column(D);
+  // Rows of a column that a thread owns: 8, 16 or 32.  What a token costs a wave beside its
+  // FMAs (two sums over the lanes, operand reads, the read-out's store) does not grow with them,
+  // so more rows mean fewer instructions in all; but a sequence and head then has fewer
+  // waves, so the most rows are taken that still leave every SIMD of the chip two waves.
+  int own = 8;
+  {
+    const long long simds = 4ll * ei_compute_units();
+    for (int wanted = 32; wanted > 8; wanted /= 2) {
+      const int lanes = lanes_a_column(D, wanted);
+      const long long waves = static_cast<long long>(n_seqs) * H *
+                              ((static_cast<long long>(DV) * lanes + EI_WAVE - 1) / EI_WAVE);
+      if (waves >= 2 * simds) {
+        own = wanted;
+        break;
+      }
+    }
+  }
+  const int L = lanes_a_column(D, own);
   const int CB = kThreads / L;
   const int C = 2 * G * D + H * DV;
   EI_REQUIRE(H <= 65535 && (DV + CB - 1) / CB <= 65535, "delta_rule: too many heads or columns");
   dim3 grid(n_seqs, H, (DV + CB - 1) / CB);
   const size_t ss = static_cast<size_t>(split_stride);
-#define EI_DELTA(TI, LL)                                                                        \
-  delta_rule_kernel<TI, LL><<<grid, kThreads, 0, stream>>>(                                     \
+#define EI_DELTA(TI, LL, OO)                                                                    \
+  delta_rule_kernel<TI, LL, OO><<<grid, kThreads, 0, stream>>>(                                 \
       conv, C, static_cast<const TI*>(proj), nsplit, ss, WP, beta_col, decay_col, a_log, dt_bias, \
       state, static_cast<size_t>(state_stride), seq_slot, seq_count, seq_row0, o_raw, H, G, D,  \
       DV, q_scale, unit_eps)
-#define EI_DELTA_L(TI)                       \
-  do {                                       \
-    if (L == 1) EI_DELTA(TI, 1);             \
-    else if (L == 2) EI_DELTA(TI, 2);        \
-    else if (L == 4) EI_DELTA(TI, 4);        \
-    else if (L == 8) EI_DELTA(TI, 8);        \
-    else if (L == 16) EI_DELTA(TI, 16);      \
-    else EI_DELTA(TI, 32);                   \
+#define EI_DELTA_O(TI, LL)                         \
+  do {                                             \
+    if (own == 8) EI_DELTA(TI, LL, 8);             \
+    else if (own == 16) EI_DELTA(TI, LL, 16);      \
+    else EI_DELTA(TI, LL, 32);                     \
+  } while (0)
+#define EI_DELTA_L(TI)                                                  \
+  do {                                                                  \
+    if (L == 1) EI_DELTA_O(TI, 1);                                      \
+    else if (L == 2) EI_DELTA_O(TI, 2);                                 \
+    else if (L == 4) EI_DELTA_O(TI, 4);                                 \
+    else if (L == 8) EI_DELTA_O(TI, 8);                                 \
+    else if (L == 16) { if (own == 8) EI_DELTA(TI, 16, 8); else EI_DELTA(TI, 16, 16); } \
+    else EI_DELTA(TI, 32, 8);                                           \
   } while (0)
   if (in_dtype == EI_F32) EI_DELTA_L(float);
   else if (in_dtype == EI_BF16) EI_DELTA_L(bf16_t);
   else EI_REQUIRE(false, "delta_rule: unknown dtype");
+#undef EI_DELTA_O
 #undef EI_DELTA_L
 #undef EI_DELTA
   EI_LAUNCH_CHECK();
