@@ -10,7 +10,10 @@ form a group with storage of its own:
                     slot the list of its pages
   state group       [entries, slots + 1, *shape] float32, zeroed when a slot is taken; the
                     last row is a spare that no sequence owns (padding of a fixed-size
-                    batch points there, so kernels need no branch for it)
+                    batch points there, so kernels need no branch for it).  A group that
+                    asks for two versions has [entries, 2 (slots + 1), *shape]: version v of
+                    slot s is row v (slots + 1) + s, and `state_version[s]` says which one
+                    holds the sequence's state; a step writes the other, and `commit` flips
 
 A slot is one live sequence.  Its length is the number of tokens it holds, which is
 also the position of its next token.  Taking a slot leaves old bytes in place: only
@@ -84,13 +87,17 @@ class SessionCache:
             self.kv_v.append(torch.empty(shape + (value_dim,), dtype=dtype, device=device))
         self._page_mirror: List[Dict[int, tuple]] = [{} for _ in self.kv_pages]
         self.states: List[torch.Tensor] = []
-        self._state_copies: List[torch.Tensor] = []     # [slots, entries, *shape], see save_states
+        # [slots, entries, *shape] (see save_states), or None for a group with two versions
+        self._state_copies: List = []
+        self.state_version = [0] * self.n_slots         # which version of a slot's rows is current
+        self.two_versions = any(request.two_versions for request, _ in layout.state_groups)
         for request, entries in layout.state_groups:
-            self.states.append(torch.zeros((len(entries), self.n_slots + 1) + tuple(request.shape),
+            rows = (2 if request.two_versions else 1) * (self.n_slots + 1)
+            self.states.append(torch.zeros((len(entries), rows) + tuple(request.shape),
                                            dtype=torch.float32, device=device))
-            self._state_copies.append(torch.empty((self.n_slots, len(entries))
-                                                  + tuple(request.shape),
-                                                  dtype=torch.float32, device=device))
+            self._state_copies.append(None if request.two_versions else torch.empty(
+                (self.n_slots, len(entries)) + tuple(request.shape), dtype=torch.float32,
+                device=device))
 
     # -- slots -------------------------------------------------------------
     def acquire(self) -> int:
@@ -98,8 +105,10 @@ class SessionCache:
         self.lengths[slot] = 0
         for pages in self.kv_pages:
             pages.open(slot)
-        for state in self.states:
+        for state, (request, _) in zip(self.states, self.layout.state_groups):
             state[:, slot].zero_()
+            if request.two_versions:
+                state[:, self.n_slots + 1 + slot].zero_()
         return slot
 
     def release(self, slot: int) -> None:
@@ -139,6 +148,20 @@ class SessionCache:
             self.lengths[slot] = new_length
             for pages in self.kv_pages:
                 pages.trim(slot, new_length)
+            if self.two_versions:         # what the step wrote is the state now
+                self.state_version[slot] ^= 1
+
+    def state_rows(self, slots: Sequence[int], n_rows: int):
+        """(rows read, rows written) in a table with two versions for a step over these slots,
+        int32 [n_rows]; rows beyond the slots are padding and name the two spare rows."""
+        spare = self.n_slots
+        rows_in = np.full(n_rows, spare, dtype=np.int32)
+        rows_out = np.full(n_rows, 2 * spare + 1, dtype=np.int32)
+        for i, slot in enumerate(slots):
+            version = self.state_version[slot]
+            rows_in[i] = version * (spare + 1) + slot
+            rows_out[i] = (1 - version) * (spare + 1) + slot
+        return rows_in, rows_out
 
     # -- fixed-size state: what a step may change in place ------------------
     def save_states(self, slots: torch.Tensor) -> None:
@@ -147,11 +170,15 @@ class SessionCache:
         and values of a failed step lie beyond the committed lengths and are simply written
         again, but state has no such place, so a failed step puts these copies back."""
         for state, copy in zip(self.states, self._state_copies):
+            if copy is None:      # two versions: the step writes the other one
+                continue
             torch.index_select(state.transpose(0, 1), 0, slots, out=copy[:slots.numel()])
 
     def restore_states(self, slots: torch.Tensor) -> None:
         """Put back what `save_states` copied for the same slots."""
         for state, copy in zip(self.states, self._state_copies):
+            if copy is None:
+                continue
             state.transpose(0, 1).index_copy_(0, slots.long(), copy[:slots.numel()])
 
     # -- views -------------------------------------------------------------
@@ -163,7 +190,8 @@ class SessionCache:
 
     def state(self, cache_id: int) -> torch.Tensor:
         """[slots + 1, *shape] float32 of a fixed-size state entry (row = slot; the last row
-        is the spare one)."""
+        is the spare one); [2 (slots + 1), *shape] for an entry with two versions (rows as
+        `meta.seq_state_in` and `meta.seq_state_out` name them)."""
         kind, group, index = self.layout.entry_group[cache_id]
         if kind != "state":
             raise KeyError(f"cache entry {cache_id} holds no fixed-size state")
@@ -188,7 +216,8 @@ class SessionCache:
     def bytes(self) -> int:
         total = 0
         for tensor in self.kv_k + self.kv_v + self.states + self._state_copies:
-            total += tensor.numel() * tensor.element_size()
+            if tensor is not None:
+                total += tensor.numel() * tensor.element_size()
         return total
 
     def check(self) -> None:

@@ -55,14 +55,16 @@ __device__ __forceinline__ float softplus_f32(float x) {
 // new_tail_state (the state again, or null): a step in which every sequence brings one row
 // may have the tails renewed here (up to kFewTaps taps), which saves the launch of delta_tail.
 // The tail of a sequence (its last J - 1 inputs before this step, oldest first) lies at
-// state + slot * state_stride + tail_offset as [J - 1, C].
+// state + row * state_stride + tail_offset as [J - 1, C]; a sequence's state is read from row
+// seq_in[seq] and written to row seq_out[seq] (the same row, or the other of two versions).
 template <typename TI>
 __global__ void delta_conv_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                                   int WP, const float* __restrict__ conv_w, int J,
                                   const float* __restrict__ state, size_t state_stride,
                                   size_t tail_offset, const int32_t* __restrict__ row_pos,
                                   const int32_t* __restrict__ row_seq,
-                                  const int32_t* __restrict__ seq_slot,
+                                  const int32_t* __restrict__ seq_in,
+                                  const int32_t* __restrict__ seq_out,
                                   const int32_t* __restrict__ seq_start, float* __restrict__ out,
                                   int C, float* __restrict__ new_tail_state) {
   const size_t row = blockIdx.x;
@@ -70,7 +72,7 @@ __global__ void delta_conv_kernel(const TI* __restrict__ proj, int nsplit, size_
   const int seq = row_seq[row];
   if (seq < 0 || c >= C) return;
   const int pos = row_pos[row], start = seq_start[seq];
-  const float* tail = state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+  const float* tail = state + static_cast<size_t>(seq_in[seq]) * state_stride + tail_offset;
   auto input = [&](int j) {                  // the input that tap j multiplies
     const int back = J - 1 - j;
     const int p = pos - back;
@@ -89,7 +91,7 @@ __global__ void delta_conv_kernel(const TI* __restrict__ proj, int nsplit, size_
     if (new_tail_state) {
       // every sequence brings this one row (the caller says so): the thread is the only
       // reader of its channel's tail, and the new tail is the inputs it holds, moved by one
-      float* to = new_tail_state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+      float* to = new_tail_state + static_cast<size_t>(seq_out[seq]) * state_stride + tail_offset;
 #pragma unroll
       for (int j = 1; j < kFewTaps; ++j)
         if (j < J) to[static_cast<size_t>(j - 1) * C + c] = x[j];
@@ -106,7 +108,8 @@ __global__ void delta_conv_kernel(const TI* __restrict__ proj, int nsplit, size_
 template <typename TI>
 __global__ void delta_tail_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                                   int WP, int J, float* __restrict__ state, size_t state_stride,
-                                  size_t tail_offset, const int32_t* __restrict__ seq_slot,
+                                  size_t tail_offset, const int32_t* __restrict__ seq_in,
+                                  const int32_t* __restrict__ seq_out,
                                   const int32_t* __restrict__ seq_count,
                                   const int32_t* __restrict__ seq_row0, int C) {
   const int seq = blockIdx.x;
@@ -114,7 +117,8 @@ __global__ void delta_tail_kernel(const TI* __restrict__ proj, int nsplit, size_
   const int count = seq_count[seq];
   if (count <= 0 || c >= C) return;          // padding of a fixed-size batch
   const size_t row = static_cast<size_t>(seq_row0[seq]) + count - 1;     // the last row
-  float* tail = state + static_cast<size_t>(seq_slot[seq]) * state_stride + tail_offset;
+  const float* tail = state + static_cast<size_t>(seq_in[seq]) * state_stride + tail_offset;
+  float* to = state + static_cast<size_t>(seq_out[seq]) * state_stride + tail_offset;
   auto kept = [&](int i) {                    // what place i of the new tail holds
     const int back = J - 2 - i;               // the input `back` positions before the last row
     return back < count ? slice_sum(proj + (row - back) * WP + c, nsplit, split_stride)
@@ -126,11 +130,11 @@ __global__ void delta_tail_kernel(const TI* __restrict__ proj, int nsplit, size_
     for (int i = 0; i < kFewTaps; ++i) keep[i] = i < J - 1 ? kept(i) : 0.f;
 #pragma unroll
     for (int i = 0; i < kFewTaps; ++i)
-      if (i < J - 1) tail[static_cast<size_t>(i) * C + c] = keep[i];
+      if (i < J - 1) to[static_cast<size_t>(i) * C + c] = keep[i];
   } else {
     float keep[kMaxTaps - 1];
     for (int i = 0; i < J - 1; ++i) keep[i] = kept(i);
-    for (int i = 0; i < J - 1; ++i) tail[static_cast<size_t>(i) * C + c] = keep[i];
+    for (int i = 0; i < J - 1; ++i) to[static_cast<size_t>(i) * C + c] = keep[i];
   }
 }
 
@@ -167,7 +171,8 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
                   size_t split_stride, int WP, int beta_col, int decay_col,
                   const float* __restrict__ a_log, const float* __restrict__ dt_bias,
                   float* __restrict__ state, size_t state_stride,
-                  const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ seq_count,
+                  const int32_t* __restrict__ seq_in, const int32_t* __restrict__ seq_out,
+                  const int32_t* __restrict__ seq_count,
                   const int32_t* __restrict__ seq_row0, float* __restrict__ o_raw, int H, int G,
                   int D, int DV, float q_scale, float unit_eps) {
   constexpr int DP = L * OWN;             // D rounded up to what the lanes of a column hold
@@ -195,8 +200,9 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
   const int i0 = part * OWN;
   const int QK = G * D, VW = H * DV;
 
-  float* mine = state + static_cast<size_t>(seq_slot[seq]) * state_stride +
-                (static_cast<size_t>(head) * DV + (col_ok ? col : 0)) * D + i0;
+  const size_t in_row = (static_cast<size_t>(head) * DV + (col_ok ? col : 0)) * D + i0;
+  const float* mine = state + static_cast<size_t>(seq_in[seq]) * state_stride + in_row;
+  float* mine_out = state + static_cast<size_t>(seq_out[seq]) * state_stride + in_row;
   // (D a multiple of 4: the rows a thread owns are whole 16-byte pieces, inside S or outside)
   const bool wide = D % 4 == 0;
   float s[OWN];
@@ -356,12 +362,12 @@ delta_rule_kernel(const float* __restrict__ conv, int C, const TI* __restrict__ 
 #pragma unroll
       for (int pc = 0; pc < PIECES; ++pc)
         if (i0 + 4 * pc < D)
-          *reinterpret_cast<float4*>(mine + 4 * pc) =
+          *reinterpret_cast<float4*>(mine_out + 4 * pc) =
               make_float4(s[4 * pc], s[4 * pc + 1], s[4 * pc + 2], s[4 * pc + 3]);
     } else {
 #pragma unroll
       for (int m = 0; m < OWN; ++m)
-        if (i0 + m < D) mine[m] = s[m];
+        if (i0 + m < D) mine_out[m] = s[m];
     }
   }
 }
@@ -406,10 +412,10 @@ int lanes_a_column(int D, int own) {
 extern "C" int ei_delta_conv(const void* proj, int in_dtype, int nsplit, long long split_stride,
                              int WP, const float* conv_w, int J, const float* state,
                              long long state_stride, long long tail_offset, const int32_t* row_pos,
-                             const int32_t* row_seq, const int32_t* seq_slot,
-                             const int32_t* seq_start, float* out, int N, int C, int renew_tail,
-                             hipStream_t stream) {
-  EI_REQUIRE(proj && conv_w && state && row_pos && row_seq && seq_slot && seq_start && out,
+                             const int32_t* row_seq, const int32_t* seq_in,
+                             const int32_t* seq_out, const int32_t* seq_start, float* out, int N,
+                             int C, int renew_tail, hipStream_t stream) {
+  EI_REQUIRE(proj && conv_w && state && row_pos && row_seq && seq_in && seq_out && seq_start && out,
              "delta_conv: null pointer");
   EI_REQUIRE(!renew_tail || J <= kFewTaps, "delta_conv: the tails are renewed here for up to 8 taps");
   float* renewed = renew_tail ? const_cast<float*>(state) : nullptr;
@@ -422,12 +428,12 @@ extern "C" int ei_delta_conv(const void* proj, int in_dtype, int nsplit, long lo
     delta_conv_kernel<float><<<grid, kThreads, 0, stream>>>(
         static_cast<const float*>(proj), nsplit, ss, WP, conv_w, J, state,
         static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
-        seq_slot, seq_start, out, C, renewed);
+        seq_in, seq_out, seq_start, out, C, renewed);
   else if (in_dtype == EI_BF16)
     delta_conv_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(
         static_cast<const bf16_t*>(proj), nsplit, ss, WP, conv_w, J, state,
         static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
-        seq_slot, seq_start, out, C, renewed);
+        seq_in, seq_out, seq_start, out, C, renewed);
   else
     EI_REQUIRE(false, "delta_conv: unknown dtype");
   EI_LAUNCH_CHECK();
@@ -435,10 +441,10 @@ extern "C" int ei_delta_conv(const void* proj, int in_dtype, int nsplit, long lo
 
 extern "C" int ei_delta_tail(const void* proj, int in_dtype, int nsplit, long long split_stride,
                              int WP, int J, float* state, long long state_stride,
-                             long long tail_offset, const int32_t* seq_slot,
-                             const int32_t* seq_count, const int32_t* seq_row0, int n_seqs, int C,
-                             hipStream_t stream) {
-  EI_REQUIRE(proj && state && seq_slot && seq_count && seq_row0, "delta_tail: null pointer");
+                             long long tail_offset, const int32_t* seq_in,
+                             const int32_t* seq_out, const int32_t* seq_count,
+                             const int32_t* seq_row0, int n_seqs, int C, hipStream_t stream) {
+  EI_REQUIRE(proj && state && seq_in && seq_out && seq_count && seq_row0, "delta_tail: null pointer");
   EI_REQUIRE(n_seqs > 0 && C > 0 && C <= WP && nsplit >= 1, "delta_tail: sizes must be positive");
   EI_REQUIRE(J >= 2 && J <= kMaxTaps, "delta_tail: taps must lie between 2 and 32");
   EI_REQUIRE((C + kThreads - 1) / kThreads <= 65535, "delta_tail: too many channels");
@@ -447,13 +453,13 @@ extern "C" int ei_delta_tail(const void* proj, int in_dtype, int nsplit, long lo
   if (in_dtype == EI_F32)
     delta_tail_kernel<float><<<grid, kThreads, 0, stream>>>(
         static_cast<const float*>(proj), nsplit, ss, WP, J, state,
-        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), seq_slot, seq_count,
-        seq_row0, C);
+        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), seq_in, seq_out,
+        seq_count, seq_row0, C);
   else if (in_dtype == EI_BF16)
     delta_tail_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(
         static_cast<const bf16_t*>(proj), nsplit, ss, WP, J, state,
-        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), seq_slot, seq_count,
-        seq_row0, C);
+        static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), seq_in, seq_out,
+        seq_count, seq_row0, C);
   else
     EI_REQUIRE(false, "delta_tail: unknown dtype");
   EI_LAUNCH_CHECK();
@@ -465,11 +471,12 @@ extern "C" int ei_delta_tail(const void* proj, int in_dtype, int nsplit, long lo
 extern "C" int ei_delta_rule(const float* conv, const void* proj, int in_dtype, int nsplit,
                              long long split_stride, int WP, int beta_col, int decay_col,
                              const float* a_log, const float* dt_bias, float* state,
-                             long long state_stride, const int32_t* seq_slot,
-                             const int32_t* seq_count, const int32_t* seq_row0, float* o_raw,
+                             long long state_stride, const int32_t* seq_in,
+                             const int32_t* seq_out, const int32_t* seq_count,
+                             const int32_t* seq_row0, float* o_raw,
                              int n_seqs, int H, int G, int D, int DV, float q_scale,
                              float unit_eps, hipStream_t stream) {
-  EI_REQUIRE(conv && proj && a_log && dt_bias && state && seq_slot && seq_count && seq_row0 && o_raw,
+  EI_REQUIRE(conv && proj && a_log && dt_bias && state && seq_in && seq_out && seq_count && seq_row0 && o_raw,
              "delta_rule: null pointer");
   EI_REQUIRE(n_seqs > 0 && H > 0 && G > 0 && H % G == 0 && DV > 0, "delta_rule: bad head counts");
   EI_REQUIRE(D >= 1 && D <= 256, "delta_rule: the key size must lie between 1 and 256");
@@ -501,7 +508,8 @@ extern "C" int ei_delta_rule(const float* conv, const void* proj, int in_dtype, 
 #define EI_DELTA(TI, LL, OO)                                                                    \
   delta_rule_kernel<TI, LL, OO><<<grid, kThreads, 0, stream>>>(                                 \
       conv, C, static_cast<const TI*>(proj), nsplit, ss, WP, beta_col, decay_col, a_log, dt_bias, \
-      state, static_cast<size_t>(state_stride), seq_slot, seq_count, seq_row0, o_raw, H, G, D,  \
+      state, static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, H, \
+      G, D,                                                                                     \
       DV, q_scale, unit_eps)
 #define EI_DELTA_O(TI, LL)                         \
   do {                                             \

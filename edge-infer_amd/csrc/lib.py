@@ -50,12 +50,14 @@ _SIGNATURES = {
     "delta_rule": {
         "ei_delta_conv": [c_void_p, c_int, c_int, c_longlong, c_int, c_void_p, c_int, c_void_p,
                           c_longlong, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_int, c_void_p],
+                          c_void_p, c_int, c_int, c_int, c_void_p],
         "ei_delta_tail": [c_void_p, c_int, c_int, c_longlong, c_int, c_int, c_void_p, c_longlong,
-                          c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+                          c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                          c_void_p],
         "ei_delta_rule": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_int, c_int, c_int,
                           c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p,
-                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
+                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float,
+                          c_void_p],
         "ei_delta_out": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_int, c_int, c_void_p,
                          c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     },
@@ -689,22 +691,30 @@ def _delta_proj(proj, rows, shape):
 
 def _delta_state(state, shape):
     if state.dim() != 2 or state.shape[1] != shape.state_floats:
-        raise KernelError(f"delta: the state must be [slots, {shape.state_floats}], "
+        raise KernelError(f"delta: the state must be [rows, {shape.state_floats}], "
                           f"got {list(state.shape)}")
     return _gpu(state, "state", torch.float32)
+
+
+def _delta_rows(seq_in, seq_out, n_seqs):
+    """A sequence's state is read from row seq_in[s] of the state table and written to row
+    seq_out[s] (the same row, or the other of two versions)."""
+    if seq_in.numel() < n_seqs or seq_out.numel() < n_seqs:
+        raise KernelError("delta: state row lists shorter than the sequences")
+    return _gpu(seq_in, "seq_in", torch.int32), _gpu(seq_out, "seq_out", torch.int32)
 
 
 DELTA_FEW_TAPS = 8      # up to so many taps `delta_conv` can renew the tails itself
 
 
-def delta_conv(proj, conv_w, state, shape: DeltaShape, row_pos, row_seq, seq_slot, seq_start,
-               out, renew_tail=False) -> None:
+def delta_conv(proj, conv_w, state, shape: DeltaShape, row_pos, row_seq, seq_in, seq_out,
+               seq_start, out, renew_tail=False) -> None:
     """out [rows, channels] float32 = silu(causal convolution) of the q, k, v columns of
     `proj` ([rows, width] or float32 slices of it); conv_w float32 [channels, taps]; inputs
-    from before this step come from the sequences' tails in `state` [slots, state_floats].
-    renew_tail: every sequence brings exactly one row (the caller vouches for it) and the
-    tails become the last taps - 1 inputs here, so `delta_tail` is not needed (at most
-    `DELTA_FEW_TAPS` taps)."""
+    from before this step come from the sequences' tails in `state` [rows, state_floats], row
+    seq_in[s] for sequence s.  renew_tail: every sequence brings exactly one row (the caller vouches for it) and the
+    tails become the last taps - 1 inputs here, written to row seq_out[s], so `delta_tail` is
+    not needed (at most `DELTA_FEW_TAPS` taps)."""
     lib = library("delta_rule")
     rows = out.shape[0]
     if tuple(out.shape) != (rows, shape.channels) or tuple(conv_w.shape) != (shape.channels, shape.taps):
@@ -717,36 +727,38 @@ def delta_conv(proj, conv_w, state, shape: DeltaShape, row_pos, row_seq, seq_slo
                                _delta_state(state, shape), shape.state_floats, shape.tail_offset,
                                _gpu(row_pos, "row_pos", torch.int32),
                                _gpu(row_seq, "row_seq", torch.int32),
-                               _gpu(seq_slot, "seq_slot", torch.int32),
+                               *_delta_rows(seq_in, seq_out, seq_start.numel()),
                                _gpu(seq_start, "seq_start", torch.int32),
                                _gpu(out, "out", torch.float32), rows, shape.channels,
                                int(bool(renew_tail)), _stream())
     _check(lib, status, "delta_conv")
 
 
-def delta_tail(proj, state, shape: DeltaShape, rows, seq_slot, seq_count, seq_row0) -> None:
-    """The sequences' tails in `state` become the last taps - 1 inputs after this step (of
-    `rows` packed rows; sequence s brings seq_count[s] of them from row seq_row0[s] on)."""
+def delta_tail(proj, state, shape: DeltaShape, rows, seq_in, seq_out, seq_count, seq_row0) -> None:
+    """The sequences' tails become the last taps - 1 inputs after this step (of `rows` packed
+    rows; sequence s brings seq_count[s] of them from row seq_row0[s] on): read from row
+    seq_in[s] of `state` where the step brought fewer, written to row seq_out[s]."""
     if shape.taps < 2:
         return
     lib = library("delta_rule")
     n_seqs = seq_count.numel()
-    if seq_slot.numel() < n_seqs or seq_row0.numel() < n_seqs:
+    if seq_row0.numel() < n_seqs:
         raise KernelError("delta_tail: sequence metadata shorter than the sequences")
     pointer, code, nsplit, stride = _delta_proj(proj, rows, shape)
     status = lib.ei_delta_tail(pointer, code, nsplit, stride, shape.width, shape.taps,
                                _delta_state(state, shape), shape.state_floats, shape.tail_offset,
-                               _gpu(seq_slot, "seq_slot", torch.int32),
+                               *_delta_rows(seq_in, seq_out, n_seqs),
                                _gpu(seq_count, "seq_count", torch.int32),
                                _gpu(seq_row0, "seq_row0", torch.int32), n_seqs, shape.channels,
                                _stream())
     _check(lib, status, "delta_tail")
 
 
-def delta_rule(conv, proj, a_log, dt_bias, state, shape: DeltaShape, seq_slot, seq_count,
+def delta_rule(conv, proj, a_log, dt_bias, state, shape: DeltaShape, seq_in, seq_out, seq_count,
                seq_row0, o_raw, q_scale: float, unit_eps: float) -> None:
-    """The recurrence over every sequence's rows of this step, in order; reads and writes S in
-    `state`; o_raw [rows, heads * value_dim] float32 receives S^T q of every row."""
+    """The recurrence over every sequence's rows of this step, in order; reads S from row
+    seq_in[s] of `state` and writes it to row seq_out[s]; o_raw [rows, heads * value_dim]
+    float32 receives S^T q of every row."""
     lib = library("delta_rule")
     rows = conv.shape[0]
     n_seqs = seq_count.numel()
@@ -754,14 +766,14 @@ def delta_rule(conv, proj, a_log, dt_bias, state, shape: DeltaShape, seq_slot, s
         raise KernelError("delta_rule: conv must be [rows, channels] and o_raw [rows, heads * value_dim]")
     if a_log.numel() != shape.n_heads or dt_bias.numel() != shape.n_heads:
         raise KernelError("delta_rule: one decay rate and bias per head")
-    if seq_slot.numel() < n_seqs or seq_row0.numel() < n_seqs:
+    if seq_row0.numel() < n_seqs:
         raise KernelError("delta_rule: sequence metadata shorter than the sequences")
     pointer, code, nsplit, stride = _delta_proj(proj, rows, shape)
     status = lib.ei_delta_rule(_gpu(conv, "conv", torch.float32), pointer, code, nsplit, stride,
                                shape.width, shape.beta_col, shape.decay_col,
                                _gpu(a_log, "a_log", torch.float32),
                                _gpu(dt_bias, "dt_bias", torch.float32), _delta_state(state, shape),
-                               shape.state_floats, _gpu(seq_slot, "seq_slot", torch.int32),
+                               shape.state_floats, *_delta_rows(seq_in, seq_out, n_seqs),
                                _gpu(seq_count, "seq_count", torch.int32),
                                _gpu(seq_row0, "seq_row0", torch.int32),
                                _gpu(o_raw, "o_raw", torch.float32), n_seqs, shape.n_heads,

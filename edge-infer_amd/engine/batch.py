@@ -10,6 +10,9 @@ in one int32 buffer of named sections:
   seq_slot[B] seq_start[B] seq_count[B]  per sequence: cache slot (its row in every state
   seq_row0[B]                          table), tokens held before the step, tokens brought,
                                        the first of its packed rows
+  seq_state_in[B] seq_state_out[B]     (models with state tables of two versions) the row of
+                                       such a table that holds the sequence's state, and the
+                                       row that the step writes
   pages<g>[B, width]                   per key/value group: logical page -> physical page
   ...                                  whatever the model's parts plan for themselves
 
@@ -52,7 +55,7 @@ class StepPlan:
     the longest sequence of the step itself."""
 
     def __init__(self, seqs: List[SeqStep], pad_seqs: Optional[int] = None,
-                 context_bound: Optional[int] = None, spare_slot: int = -1):
+                 context_bound: Optional[int] = None, spare_slot: int = -1, state_rows=None):
         if not seqs:
             raise ValueError("a step needs at least one sequence")
         self.seqs = seqs
@@ -124,6 +127,10 @@ class StepPlan:
             want_rows = [seq.row0 for seq in seqs] + [-1] * (self.n_seqs - len(seqs))
         self.want_rows = np.asarray(want_rows, dtype=np.int32)
         self.extra: Dict[str, np.ndarray] = {}
+        # (rows read, rows written) of state tables with two versions, from a function of
+        # (slots, number of sequences with padding); None: the model has no such table
+        self.state_rows = None if state_rows is None else state_rows(
+            [seq.slot for seq in seqs], self.n_seqs)
 
     def add_sections(self, sections: Mapping[str, np.ndarray]) -> None:
         """Sections that a part planned for itself.  Parts of one kind may plan the same
@@ -142,6 +149,8 @@ class StepPlan:
                ("want_rows", self.want_rows), ("seq_slot", self.seq_slot),
                ("seq_start", self.seq_start), ("seq_count", self.seq_count),
                ("seq_row0", self.seq_row0)]
+        if self.state_rows is not None:
+            out += [("seq_state_in", self.state_rows[0]), ("seq_state_out", self.state_rows[1])]
         for index, table in enumerate(page_tables):
             out.append((f"pages{index}", table.reshape(-1)))
         for name, array in self.extra.items():
@@ -240,6 +249,8 @@ class DeviceMeta:
     seq_start = property(lambda self: self.section("seq_start"))
     seq_count = property(lambda self: self.section("seq_count"))
     seq_row0 = property(lambda self: self.section("seq_row0"))
+    seq_state_in = property(lambda self: self.section("seq_state_in"))
+    seq_state_out = property(lambda self: self.section("seq_state_out"))
 
     def page_table(self, group: int) -> torch.Tensor:
         return self.section(f"pages{group}").view(self.n_seqs, self._table_widths[group])

@@ -272,8 +272,9 @@ class Session:
             else:
                 plan, meta, workspace = captured.plan, captured.meta, captured.workspace
             ctx = self._context(plan, meta, workspace, fixed_shape=captured is not None)
-            if self.cache.states:
+            if any(copy is not None for copy in self.cache._state_copies):
                 # state of fixed size is updated in place: keep what the step may change
+                # (tables with two versions need no copy: a step writes the other version)
                 saved = meta.seq_slot[:plan.n_live_seqs]
                 self.cache.save_states(saved)
             logits = (self.model.forward(ctx) if captured is None
@@ -307,7 +308,8 @@ class Session:
 
     def _plan(self, seqs, pad_seqs=None, bound=None) -> StepPlan:
         plan = StepPlan(seqs, pad_seqs=pad_seqs, context_bound=bound,
-                        spare_slot=self.cache.n_slots)
+                        spare_slot=self.cache.n_slots,
+                        state_rows=self.cache.state_rows if self.cache.two_versions else None)
         self.model.plan_step(plan)      # the parts add the sections they plan for themselves
         return plan
 

@@ -37,8 +37,16 @@ class KVRequest:
 
 @dataclass(frozen=True)
 class StateRequest:
-    """A float32 tensor of fixed shape per sequence, zero when the sequence starts."""
+    """A float32 tensor of fixed shape per sequence, zero when the sequence starts.
+
+    `two_versions` False: one row a slot, which the mixer updates in place; the session copies
+    the rows of a step's slots aside before the step and puts them back if it fails.
+    `two_versions` True (for large states): two rows a slot; a step reads the row its sequence's
+    state is in (`meta.seq_state_in`) and writes the whole other row (`meta.seq_state_out`),
+    and the two change places when the step is committed, so a failed step leaves the state as
+    it was and nothing is ever copied.  The table is then [2 (slots + 1), *shape]."""
     shape: Tuple[int, ...]
+    two_versions: bool = False
 
 
 class Workspace:

@@ -14,7 +14,9 @@ mixer's input (all of the recurrence in float32):
 The six input projections are one fused matrix [q | k | v | beta | decay | gate].  Per
 sequence the cache holds one float32 row (`StateRequest`): S of every head, then the last
 taps - 1 inputs of every convolved channel, so a prompt may arrive whole, in portions of
-any size or token by token.  Kernels: `csrc/delta_rule.hip`.
+any size or token by token.  The row has two versions: a step reads one and writes the whole
+other one, and the session makes that one current when the step is committed, so a failed
+step costs nothing and no copy of the state is ever taken.  Kernels: `csrc/delta_rule.hip`.
 """
 from __future__ import annotations
 
@@ -63,7 +65,8 @@ class GatedDelta:
 
     @classmethod
     def cache_request(cls, spec):
-        return StateRequest(shape=(cls.shape_of(spec).state_floats,))
+        # (S is a megabyte a layer and sequence at real sizes: two versions instead of copies)
+        return StateRequest(shape=(cls.shape_of(spec).state_floats,), two_versions=True)
 
     @classmethod
     def kernel_libraries(cls, spec, dtype):
@@ -100,20 +103,26 @@ class GatedDelta:
         self.q_scale = float(spec.key_dim) ** -0.5
 
     def forward(self, ctx, x, entry):
+        if not entry.writes_cache:
+            raise ValueError("gated_delta: a run that only reads another run's state is not "
+                             "implemented")
         shape, meta = self.shape, ctx.meta
         n = x.shape[0]
-        state = ctx.cache.state(entry.cache)                 # [slots + 1, state_floats]
+        state = ctx.cache.state(entry.cache)                 # [2 (slots + 1), state_floats]
+        rows_in = meta.seq_state_in                          # a sequence's state, and the row
+        rows_out = meta.seq_state_out                        # the step writes
         proj = self.proj.forward(ctx, x, "delta.proj")
         conv = ctx.buffer("delta.conv", (n, shape.channels), torch.float32)
         # a decode step (one row a sequence) renews the convolution's tails in the same kernel
-        renew = ctx.decode and entry.writes_cache and shape.taps <= lib.DELTA_FEW_TAPS
+        renew = ctx.decode and shape.taps <= lib.DELTA_FEW_TAPS
         lib.delta_conv(proj, self.conv_w, state, shape, meta.row_pos, meta.row_seq,
-                       meta.seq_slot, meta.seq_start, conv, renew_tail=renew)
-        if entry.writes_cache and not renew:
-            lib.delta_tail(proj, state, shape, n, meta.seq_slot, meta.seq_count, meta.seq_row0)
+                       rows_in, rows_out, meta.seq_start, conv, renew_tail=renew)
+        if not renew:
+            lib.delta_tail(proj, state, shape, n, rows_in, rows_out, meta.seq_count,
+                           meta.seq_row0)
         o_raw = ctx.buffer("delta.o_raw", (n, shape.v_width), torch.float32)
         lib.delta_rule(conv, proj, self.decay_log_rate, self.decay_bias, state, shape,
-                       meta.seq_slot, meta.seq_count, meta.seq_row0, o_raw, self.q_scale,
+                       rows_in, rows_out, meta.seq_count, meta.seq_row0, o_raw, self.q_scale,
                        self.spec.unit_eps)
         ctx.release(conv)
         gated = ctx.buffer("delta.gated", (n, shape.v_width))

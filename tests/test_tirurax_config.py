@@ -106,7 +106,8 @@ def test_cache_requests():
     assert kv == [KVRequest(2, 16, None, 24, 24), KVRequest(2, 32, None, None, None)]
     states = [request for request, _ in layout.state_groups]
     # 4 heads x 8 x 16 + 2 taps kept x (2 x 4 x 16 + 4 x 8);  4 x 16 x 24 + 1 x (2 x 24 + 64)
-    assert states == [StateRequest((512 + 2 * 160,)), StateRequest((1536 + 112,))]
+    assert states == [StateRequest((512 + 2 * 160,), two_versions=True),
+                      StateRequest((1536 + 112,), two_versions=True)]
 
 
 def test_pages_behind_a_chunk_go_back():

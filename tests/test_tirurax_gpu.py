@@ -170,6 +170,43 @@ def test_long_decoding_from_the_first_token(models, weights, name, dtype):
         assert (name, dtype) == ("B", "bfloat16")
 
 
+@pytest.mark.parametrize("graphs", [True, False])
+def test_a_failed_step_leaves_the_state_as_it_was(models, references, graphs):
+    """The delta layers' state has two versions a slot: a step that fails after its layers have
+    run (here the head raises, once in a prompt portion and once in a decode step) has written
+    the other version only, so the same step again gives what a run without the failure gives;
+    no copy of the state is kept for it."""
+    import edge_infer_amd as ei
+    model = models("A", "float32")
+    request, ref = requests_for("A")[0], references["A"][0]
+    session = ei.Session(model, max_tokens=512, graphs=graphs)
+    assert session.cache.two_versions and all(c is None for c in session.cache._state_copies)
+    slot = session.begin()
+    rows = [session.step([(slot, request[:40], list(range(40)))])]
+    whole = type(model).logits
+    failures = []
+
+    def failing(self, ctx, hidden):
+        if not failures:
+            failures.append(ctx.n_rows)
+            raise RuntimeError("forced failure after the layers have run")
+        return whole(self, ctx, hidden)
+    try:
+        type(model).logits = failing
+        with pytest.raises(RuntimeError, match="forced failure"):
+            session.step([(slot, request[40:90], list(range(50)))])
+        assert session.length(slot) == 40
+        rows.append(session.step([(slot, request[40:90], list(range(50)))]))
+        failures.clear()       # (the first decode step: the one that runs eagerly before a graph is made)
+        with pytest.raises(RuntimeError, match="forced failure"):
+            session.step([(slot, request[90:91], [0])])
+        for t in range(90, 100):
+            rows.append(session.step([(slot, request[t:t + 1], [0])]))
+    finally:
+        type(model).logits = whole
+    close("float32", torch.cat(rows), ref[:100], "after failed steps")
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_a_token_far_back_shows(tmp_path, name):
     """Delta layers that forget slowly: two prompts that differ in their third token alone
