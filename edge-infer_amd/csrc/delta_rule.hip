@@ -18,8 +18,8 @@
 //   delta_conv   convolution + silu of all q, k, v channels of every row
 //   delta_tail   the new last J - 1 inputs of every sequence (after delta_conv has read the
 //                old ones)
-//   delta_rule   the recurrence; a thread owns 8 rows of one column of S, L = D / 8 lanes
-//                share a column; tokens come in tiles through LDS
+//   delta_rule   the recurrence; a thread owns 8 or 16 rows of one column of S, L lanes share a
+//                column; tokens come in tiles through LDS
 //   delta_out    the read-out's norm and gate
 #include "common.h"
 
@@ -159,7 +159,7 @@ __device__ __forceinline__ float group_sum(float v) {
 
 // conv: [N, C] = q [G * D] | k [G * D] | v [H * DV] after convolution and silu.  The block
 // (sequence, head, column block) walks the sequence's rows of this step in order.  A thread owns
-// OWN rows of one column of S, L neighbouring lanes share the column.  Per token, with S the
+// OWN (8 or 16) rows of one column of S, L neighbouring lanes share the column.  Per token, with S the
 // state before the token, g its decay, k, q the unit key and the scaled unit query:
 //   seen = g (S^T k)[col];  u = beta (v[col] - seen);  o[col] = g (S^T q)[col] + u (k . q);
 //   S[., col] <- g S[., col] + k u
@@ -482,14 +482,16 @@ extern "C" int ei_delta_rule(const float* conv, const void* proj, int in_dtype, 
   EI_REQUIRE(D >= 1 && D <= 256, "delta_rule: the key size must lie between 1 and 256");
   EI_REQUIRE(beta_col >= 0 && decay_col >= 0 && beta_col + H <= WP && decay_col + H <= WP,
              "delta_rule: projection columns outside the row");
-  // Rows of a column that a thread owns: 8, 16 or 32.  What a token costs a wave beside its
-  // FMAs (two sums over the lanes, operand reads, the read-out's store) does not grow with them,
-  // so more rows mean fewer instructions in all; but a sequence and head then has fewer
-  // waves, so the most rows are taken that still leave every SIMD of the chip two waves.
+  // Rows of a column that a thread owns: 8 or 16.  What a token costs a wave beside its FMAs
+  // (two sums over the lanes, operand reads, the read-out's store) does not grow with them, so
+  // more rows mean fewer instructions in all; but a sequence and head then has fewer waves, so
+  // 16 are taken only where that still leaves every SIMD of the chip two waves.  (32 rows, 256
+  // registers and one wave a SIMD, measured slower: 2.9 against 2.5 ms for 64 prompts of 512
+  // tokens, 67 against 60 us for a decode step of 64.)
   int own = 8;
   {
     const long long simds = 4ll * ei_compute_units();
-    for (int wanted = 32; wanted > 8; wanted /= 2) {
+    for (int wanted = 16; wanted > 8; wanted /= 2) {
       const int lanes = lanes_a_column(D, wanted);
       const long long waves = static_cast<long long>(n_seqs) * H *
                               ((static_cast<long long>(DV) * lanes + EI_WAVE - 1) / EI_WAVE);
@@ -514,8 +516,7 @@ extern "C" int ei_delta_rule(const float* conv, const void* proj, int in_dtype, 
 #define EI_DELTA_O(TI, LL)                         \
   do {                                             \
     if (own == 8) EI_DELTA(TI, LL, 8);             \
-    else if (own == 16) EI_DELTA(TI, LL, 16);      \
-    else EI_DELTA(TI, LL, 32);                     \
+    else EI_DELTA(TI, LL, 16);                     \
   } while (0)
 #define EI_DELTA_L(TI)                                                  \
   do {                                                                  \
@@ -523,7 +524,7 @@ extern "C" int ei_delta_rule(const float* conv, const void* proj, int in_dtype, 
     else if (L == 2) EI_DELTA_O(TI, 2);                                 \
     else if (L == 4) EI_DELTA_O(TI, 4);                                 \
     else if (L == 8) EI_DELTA_O(TI, 8);                                 \
-    else if (L == 16) { if (own == 8) EI_DELTA(TI, 16, 8); else EI_DELTA(TI, 16, 16); } \
+    else if (L == 16) EI_DELTA_O(TI, 16);                               \
     else EI_DELTA(TI, 32, 8);                                           \
   } while (0)
   if (in_dtype == EI_F32) EI_DELTA_L(float);
