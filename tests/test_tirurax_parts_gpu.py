@@ -248,14 +248,17 @@ def plain_delta(params, mixer, x):
     return plain.delta_mixer(x, p, m, mixer.out_norm_eps)
 
 
-@pytest.mark.parametrize("variant", ["base", "one tap", "wide keys", "odd sizes", "many taps"])
+@pytest.mark.parametrize("variant", ["base", "one tap", "wide keys", "odd sizes", "many taps",
+                                     "ten taps", "keys of 256"])
 def test_delta_rule_alone(variant):
     """Two sequences: whole prompts of unequal lengths, then portions of 2, 1 and 5 rows, then
     single tokens; the state and the convolution's tail carry over every cut."""
     kw = {"base": {}, "one tap": dict(conv_taps=1, n_heads=2, n_kv_heads=2, key_dim=8, value_dim=8),
           "wide keys": dict(key_dim=144, value_dim=12, n_heads=2, n_kv_heads=1),
           "odd sizes": dict(key_dim=13, value_dim=5, n_heads=3, n_kv_heads=1, conv_taps=2),
-          "many taps": dict(conv_taps=7, key_dim=64, value_dim=64, n_heads=2, n_kv_heads=2)}[variant]
+          "many taps": dict(conv_taps=7, key_dim=64, value_dim=64, n_heads=2, n_kv_heads=2),
+          "ten taps": dict(conv_taps=10, key_dim=16, value_dim=24, n_heads=2, n_kv_heads=1),
+          "keys of 256": dict(key_dim=256, value_dim=8, n_heads=1, n_kv_heads=1, conv_taps=3)}[variant]
     mixer = delta_spec(**kw)
     spec = one_layer(mixer)
     params = params_for(spec, 8)
