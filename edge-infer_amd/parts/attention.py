@@ -33,6 +33,9 @@ from .linear import Linear
 # EDGE_INFER_FUSED_DECODE=0: decode steps launch the norm-rotate-store kernel of their own
 # instead of letting the matrix-core decode kernel do that work
 FUSED_DECODE = os.environ.get("EDGE_INFER_FUSED_DECODE", "1") != "0"
+# EDGE_INFER_MATRIX_CORE_ATTENTION=0: bfloat16 attention runs on the generic kernel (float32
+# arithmetic on the cached bfloat16 keys and values) whatever the head size
+MATRIX_CORE_ATTENTION = os.environ.get("EDGE_INFER_MATRIX_CORE_ATTENTION", "1") != "0"
 
 
 # What the matrix-core decode kernel costs, measured on an MI355X: a wave walks a tile of 16
@@ -102,7 +105,7 @@ class Attention:
         """What this part will run, so that a model can have it compiled ahead of its first
         step."""
         group = spec.n_heads // max(1, spec.n_kv_heads)
-        fast = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim
+        fast = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and MATRIX_CORE_ATTENTION
                 and lib.attention_decode_mfma_supported(spec.head_dim, group))
         return ("rope_store", "attention_mfma" if fast else "attention_generic",
                 *Linear.kernel_libraries(dtype))
@@ -170,6 +173,7 @@ class Attention:
         # the matrix-core kernels take bfloat16 with head sizes 64 and 128 and values as wide
         # as the keys; every other case runs the generic kernel
         self.matrix_cores = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and
+                            MATRIX_CORE_ATTENTION and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
         # chunk, slopes, sink: what the kernels take beyond a window
         self.extras = dict(chunk=spec.chunk, slopes=self.slopes, sinks=self.sinks)
