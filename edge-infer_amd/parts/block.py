@@ -4,6 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..csrc import lib
+from ..weights.loader import ParamSpec
 from .registry import lookup
 
 
@@ -110,6 +111,12 @@ class OutputNormBlock:
         for prefix, owner, spec in cls._owners(layer_spec):
             for name, param in owner.parameters(spec, hidden).items():
                 params[f"{prefix}.{name}"] = param
+        if layer_spec.feed_forward is None:
+            # a checkpoint may still hold the second norm of a layer without a feed-forward;
+            # it is taken and has no use
+            norm_cls = lookup("norm", layer_spec.norm.kind)
+            for name, param in norm_cls.parameters(layer_spec.norm, hidden).items():
+                params[f"norm2.{name}"] = ParamSpec(param.shape, init=param.init, optional=True)
         return params
 
     @classmethod

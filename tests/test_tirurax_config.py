@@ -79,6 +79,18 @@ def test_weights_that_do_not_fit_are_named():
     assert error.value.missing == ["l0.mix.sink"] and error.value.unexpected == ["l1.mix.extra"]
 
 
+def test_a_second_norm_without_a_feed_forward_is_taken_and_unused():
+    from edge_infer_amd.engine.model import expected_parameters
+    from edge_infer_amd.weights import match_parameters
+    cfg = config("A")
+    expected = expected_parameters(cfg.model_spec(), cfg.checkpoint_name)
+    tensors = sharp_weights(CONFIGS["A"], 0)
+    assert "l1.norm2" not in tensors                 # layer 1 has no feed-forward
+    matched = match_parameters(expected, tensors)
+    tensors["l1.norm2"] = torch.ones(CONFIGS["A"]["width"])
+    assert len(match_parameters(expected, tensors)) == len(matched) + 1
+
+
 @pytest.mark.parametrize("change, message", [
     (lambda c: c["layers"][0].update(type="conv"), "type"),
     (lambda c: c["layers"][0]["mixer"].update(window=5), "does not know"),
