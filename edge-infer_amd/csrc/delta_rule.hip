@@ -102,6 +102,70 @@ __global__ void delta_conv_kernel(const TI* __restrict__ proj, int nsplit, size_
   out[row * C + c] = silu_f32(acc);
 }
 
+// The same for four neighbouring channels a thread (channel counts, row widths and slice
+// strides that are multiples of 4, up to kFewTaps taps): 8- or 16-byte loads of the inputs, the
+// filters of four channels as J consecutive 16-byte pieces, one 16-byte store.
+template <typename TI>
+__global__ void delta_conv_vec_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
+                                      int WP, const float* __restrict__ conv_w, int J,
+                                      const float* __restrict__ state, size_t state_stride,
+                                      size_t tail_offset, const int32_t* __restrict__ row_pos,
+                                      const int32_t* __restrict__ row_seq,
+                                      const int32_t* __restrict__ seq_in,
+                                      const int32_t* __restrict__ seq_out,
+                                      const int32_t* __restrict__ seq_start,
+                                      float* __restrict__ out, int C,
+                                      float* __restrict__ new_tail_state) {
+  const size_t row = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+  const int seq = row_seq[row];
+  if (seq < 0 || c >= C) return;
+  const int pos = row_pos[row], start = seq_start[seq];
+  const float* tail = state + static_cast<size_t>(seq_in[seq]) * state_stride + tail_offset;
+  float x[kFewTaps][4];
+#pragma unroll
+  for (int j = 0; j < kFewTaps; ++j) {
+    x[j][0] = x[j][1] = x[j][2] = x[j][3] = 0.f;
+    if (j < J) {
+      const int back = J - 1 - j;
+      const int p = pos - back;
+      if (p >= start) {
+        const TI* src = proj + (row - back) * WP + c;
+        for (int s0 = 0; s0 < nsplit; s0 += 4) {
+          float v[4][4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (s0 + u < nsplit) ei::Vec4<TI>::load(src + (s0 + u) * split_stride, v[u]);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (s0 + u < nsplit) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) x[j][e] += v[u][e];
+            }
+        }
+      } else if (p >= 0) {
+        ei::Vec4<float>::load(tail + static_cast<size_t>(p - start + J - 1) * C + c, x[j]);
+      }
+    }
+  }
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < kFewTaps; ++j)
+    if (j < J) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] += conv_w[static_cast<size_t>(c + e) * J + j] * x[j][e];
+    }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) acc[e] = silu_f32(acc[e]);
+  ei::Vec4<float>::store(out + row * C + c, acc);
+  if (new_tail_state) {
+    float* to = new_tail_state + static_cast<size_t>(seq_out[seq]) * state_stride + tail_offset;
+#pragma unroll
+    for (int j = 1; j < kFewTaps; ++j)
+      if (j < J) ei::Vec4<float>::store(to + static_cast<size_t>(j - 1) * C + c, x[j]);
+  }
+}
+
 // A thread writes a sequence's new tail for its channel: the inputs of the last J - 1
 // positions, from this step's rows or, where the step brought fewer, from the old tail (read
 // before anything is written).
@@ -424,6 +488,27 @@ extern "C" int ei_delta_conv(const void* proj, int in_dtype, int nsplit, long lo
   EI_REQUIRE((C + kThreads - 1) / kThreads <= 65535, "delta_conv: too many channels");
   const dim3 grid(N, (C + kThreads - 1) / kThreads);
   const size_t ss = static_cast<size_t>(split_stride);
+  const bool vec = J <= kFewTaps && C % 4 == 0 && WP % 4 == 0 && ss % 4 == 0 &&
+                   state_stride % 4 == 0 && tail_offset % 4 == 0 &&
+                   (reinterpret_cast<uintptr_t>(proj) | reinterpret_cast<uintptr_t>(out) |
+                    reinterpret_cast<uintptr_t>(state)) % 16 == 0;
+  if (vec) {
+    const int threads = 64;         // four channels a thread: 256 channels a block
+    const dim3 vgrid(N, (C / 4 + threads - 1) / threads);
+    if (in_dtype == EI_F32)
+      delta_conv_vec_kernel<float><<<vgrid, threads, 0, stream>>>(
+          static_cast<const float*>(proj), nsplit, ss, WP, conv_w, J, state,
+          static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
+          seq_in, seq_out, seq_start, out, C, renewed);
+    else if (in_dtype == EI_BF16)
+      delta_conv_vec_kernel<bf16_t><<<vgrid, threads, 0, stream>>>(
+          static_cast<const bf16_t*>(proj), nsplit, ss, WP, conv_w, J, state,
+          static_cast<size_t>(state_stride), static_cast<size_t>(tail_offset), row_pos, row_seq,
+          seq_in, seq_out, seq_start, out, C, renewed);
+    else
+      EI_REQUIRE(false, "delta_conv: unknown dtype");
+    EI_LAUNCH_CHECK();
+  }
   if (in_dtype == EI_F32)
     delta_conv_kernel<float><<<grid, kThreads, 0, stream>>>(
         static_cast<const float*>(proj), nsplit, ss, WP, conv_w, J, state,
