@@ -1,5 +1,5 @@
-"""edge-infer for AMD MI355X: a small generation library for the Qwen3 dense and the Tirurax
-decoders (the architecture is the one that a folder's config.json names).
+"""edge-infer for AMD MI355X: a small generation library for the Qwen3 dense, the Tirurax and
+the Zadenex decoders (the architecture is the one that a folder's config.json names).
 
     model = load_model("/path/to/folder", dtype="bfloat16")     # config.json + safetensors
     session = Session(model, max_tokens=4096)
@@ -11,7 +11,8 @@ Importing the package needs no GPU; building a model or a session does.
 from __future__ import annotations
 
 from . import config, parts  # registers the built-in architecture and parts
-from .config import Qwen3Config, TiruraxConfig, read_config, register_architecture
+from .config import (Qwen3Config, TiruraxConfig, ZadenexConfig, read_config,
+                     register_architecture)
 from .weights import WeightsError, write_model_folder
 
 __version__ = "0.1.0"

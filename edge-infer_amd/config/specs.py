@@ -22,7 +22,9 @@ class NormSpec:
 @dataclass(frozen=True)
 class PositionSpec:
     """Position encoding of a mixer.  kind "rope": rotate-half pairs (i, i+dim/2)
-    with angle = position / theta^(2i/dim); kind "none": no encoding."""
+    with angle = position / theta^(2i/dim), from a table of `max_positions` rows; kind
+    "rope_pairs": neighbouring pairs (2i, 2i+1) with the same angles, worked out by the kernels
+    from the frequencies theta^(-2i/dim), so no position is too far; kind "none": no encoding."""
     kind: str = "rope"
     theta: float = 10000.0
     dim: int = 0
@@ -57,6 +59,15 @@ class AttentionSpec:
     # a learned number per head that joins the softmax's denominator as exp(sink), with no
     # key and no value
     sink: bool = False
+    # the softmax's denominator holds a 1 besides the keys' terms (a sink of score 0 that is
+    # not learned); not together with `sink`
+    unit_sink: bool = False
+    # a learned matrix T [heads, heads] mixes the scaled scores of a (query, key) pair over the
+    # heads before the softmax: score_h <- sum_g T[h, g] score_g
+    talking_heads: bool = False
+    # the output projection's bias: None: taken when the checkpoint holds it, True: it must
+    # hold it, False: it must not
+    o_bias: Optional[bool] = None
 
     @property
     def q_width(self) -> int:
@@ -97,6 +108,60 @@ class DenseMLPSpec:
 
 
 @dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Causal attention whose keys and values are up-projections of one latent vector a
+    position, which is all the cache holds besides one rotated key part that every head
+    shares.  Queries pass a normed latent of their own.  A head's query and key are
+    [head_dim unrotated | rot_dim rotated].  See `parts.latent`."""
+    kind: str = "latent_attention"
+    n_heads: int = 0
+    head_dim: int = 0             # unrotated query/key elements of a head
+    rot_dim: int = 0              # rotated elements of a head; the key's are shared by all heads
+    value_dim: int = 0
+    kv_rank: int = 0              # width of the cached latent
+    q_rank: int = 0               # width of the queries' latent
+    scale: Optional[float] = None         # None: 1/sqrt(head_dim + rot_dim)
+    norm_eps: float = 1e-6                # eps of the RMS norms of the two latents
+    position: PositionSpec = field(default_factory=lambda: PositionSpec(kind="rope_pairs"))
+    sink: bool = False            # a learned number per head in the softmax's denominator
+    output_gate: bool = False     # a head's output is multiplied by sigmoid(w_h . x), x the input
+
+    @property
+    def q_width(self) -> int:
+        return self.n_heads * (self.head_dim + self.rot_dim)
+
+    @property
+    def cache_width(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+    @property
+    def out_width(self) -> int:
+        return self.n_heads * self.value_dim
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """Matrix memory with exponential gates (mLSTM): a recurrent mixer whose state is one
+    [key_dim, value_dim] matrix, a normaliser [key_dim] and a running maximum per head.  See
+    `parts.mlstm`."""
+    kind: str = "mlstm"
+    n_heads: int = 0
+    key_dim: int = 0
+    value_dim: int = 0
+    gate_cap: float = 15.0        # the gates' pre-activations pass cap * tanh(x / cap)
+    out_norm_eps: float = 1e-6    # eps of the RMS norm of each head's read-out
+    bottom_eps: float = 1e-6      # added to the read-out's denominator
+
+    @property
+    def qk_width(self) -> int:
+        return self.n_heads * self.key_dim
+
+    @property
+    def v_width(self) -> int:
+        return self.n_heads * self.value_dim
+
+
+@dataclass(frozen=True)
 class GatedDeltaSpec:
     """Gated delta rule: a recurrent mixer whose state is one [key_dim, value_dim] matrix per
     head, fed through short causal convolutions.  See `parts.delta`."""
@@ -124,6 +189,19 @@ class LayerSpec:
     norm: NormSpec
     mixer: object         # a spec with a .kind (AttentionSpec, or one a test registers)
     feed_forward: object  # a spec with a .kind (GatedMLPSpec, ...), or None: no feed-forward
+    # what a sublayer adds to the stream is multiplied by this (arrangements that know it)
+    residual_scale: float = 1.0
+
+
+@dataclass(frozen=True)
+class LoopSpec:
+    """Layers start .. stop - 1 run `times` times in a row with the same weights, each pass
+    with cache entries of its own.  Before a pass the stream x is made anew from itself and the
+    embedding output x0: x <- W [x ; x0] + step[pass], with W [hidden, 2 hidden] and step
+    [times, hidden] parameters of the model."""
+    start: int
+    stop: int
+    times: int
 
 
 @dataclass(frozen=True)
@@ -147,6 +225,8 @@ class ModelSpec:
     max_position_embeddings: int
     bos_token_id: Optional[int]   # None: the architecture names no such token
     eos_token_id: Optional[int]
+    embedding_scale: float = 1.0         # the embedding rows are multiplied by this
+    loop: Optional[LoopSpec] = None      # the schedule then has to be `looped_schedule`'s
 
     def validate(self) -> None:
         if not self.layers or not self.schedule:
@@ -159,6 +239,13 @@ class ModelSpec:
                 if entry.cache in writers:
                     raise ValueError(f"cache entry {entry.cache} has two writers")
                 writers[entry.cache] = entry.layer
+        if self.loop is not None:
+            loop = self.loop
+            if not (0 <= loop.start < loop.stop <= len(self.layers)) or loop.times < 1:
+                raise ValueError(f"a loop over layers {loop.start}..{loop.stop - 1}, {loop.times} "
+                                 f"times, does not fit {len(self.layers)} layers")
+            if self.schedule != looped_schedule(len(self.layers), loop):
+                raise ValueError("the schedule of a model with a loop must be looped_schedule's")
         seen = set()
         for entry in self.schedule:
             if entry.writes_cache:
@@ -171,3 +258,18 @@ class ModelSpec:
 def default_schedule(n_layers: int) -> Tuple[ScheduleEntry, ...]:
     """Every layer once, in order, each with a cache entry of its own."""
     return tuple(ScheduleEntry(layer=i, cache=i) for i in range(n_layers))
+
+
+def looped_schedule(n_layers: int, loop: LoopSpec) -> Tuple[ScheduleEntry, ...]:
+    """The layers before the loop, the looped layers `times` times, the rest; every run has a
+    cache entry of its own."""
+    order = list(range(loop.start))
+    for _ in range(loop.times):
+        order += list(range(loop.start, loop.stop))
+    order += list(range(loop.stop, n_layers))
+    return tuple(ScheduleEntry(layer=layer, cache=run) for run, layer in enumerate(order))
+
+
+def pass_starts(n_layers: int, loop: LoopSpec):
+    """Index in `looped_schedule` of the first run of every pass."""
+    return tuple(loop.start + t * (loop.stop - loop.start) for t in range(loop.times))

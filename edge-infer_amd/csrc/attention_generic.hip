@@ -1,5 +1,5 @@
-// Causal grouped-query attention over the paged cache, any key and value head size up to
-// 256 (the two may differ), any head and group counts, float32 or bfloat16
+// Causal grouped-query attention over the paged cache, any key head size up to 1024 and value
+// head size up to 512 (the two may differ), any head and group counts, float32 or bfloat16
 // storage, float32 arithmetic throughout (scores, running maximum, exponentials,
 // sums and the value accumulation).  One kernel serves prefill (many positions of a
 // sequence) and decode (one position, the key range split over several blocks and
@@ -10,7 +10,12 @@
 // o = sum w_t v_t / sum w_t; query head h reads kv head h / (nq / nkv).
 // Options beyond the reference: `chunk` (a query at p sees key t only if t / chunk == p / chunk),
 // `slopes` (per query head: the score is lowered by slope * (p - t)), `sinks` (per query head:
-// exp(sink) joins the denominator; it has no key and no value).
+// exp(sink) joins the denominator; it has no key and no value), `key_heads` (a query row is
+// key_heads * D wide and meets the keys of all kv heads of a position laid end to end, which is
+// how scores mixed over heads are taken: a mix of scores is the score of mixed queries;
+// values still come from the row's own kv head), `values_in_keys` (the values are the first DV
+// elements of the key rows: a latent that serves as key and value is cached once), `gate` (per
+// row and head: the output is multiplied by sigmoid(gate)).
 // operators/src/cuda/execution.cu:137-179, runtime/src/qwen.cpp:374-402,
 // split merge: operators/src/cuda/kernels/gather_fa_variable.cu:14-118.
 #include "common.h"
@@ -20,6 +25,7 @@ namespace {
 constexpr int kRows = 16;     // query rows (positions x heads of one kv group) per block
 constexpr int kThreads = 256;
 constexpr float kLowest = -1.0e30f;
+constexpr int kAcc = 32;      // a lane holds every 16th value element: values up to 16 * kAcc wide
 
 // Work item: `npos` consecutive packed rows starting at `row0`, all of sequence `seq`.
 template <typename T>
@@ -32,11 +38,13 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                     float* __restrict__ part_ml, int nq, int nkv, int D, int DV, int Gb,
                     int head_blocks, int BC, int window, int chunk,
                     const float* __restrict__ slopes, const float* __restrict__ sinks,
-                    float scale, int n_splits) {
+                    float scale, int n_splits, int KH, int values_in_keys,
+                    const float* __restrict__ gate) {
   extern __shared__ float lds[];
-  float* Qs = lds;                        // [kRows][D]
-  float* Ks = Qs + kRows * D;             // [BC][D + 1]
-  float* Vs = Ks + BC * (D + 1);          // [BC][DV]
+  const int DQ = KH * D;                  // width of a query row and of a key as it is met
+  float* Qs = lds;                        // [kRows][DQ]
+  float* Ks = Qs + kRows * DQ;            // [BC][DQ + 1]
+  float* Vs = Ks + BC * (DQ + 1);         // [BC][DV]
   float* Ps = Vs + BC * DV;               // [kRows][BC + 1]
 
   const int item = blockIdx.x;
@@ -58,19 +66,19 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
   const int chunk_r = (chunk > 0 && row_valid) ? pos_r / chunk : 0;
 
   // query rows, pre-scaled
-  for (int idx = t; idx < kRows * D; idx += kThreads) {
-    const int rr = idx / D, d = idx % D;
+  for (int idx = t; idx < kRows * DQ; idx += kThreads) {
+    const int rr = idx / DQ, d = idx % DQ;
     const int ppi = rr / Gb, hhi = hb * Gb + rr % Gb;
     float v = 0.f;
     if (seq >= 0 && ppi < npos && hhi < G)
-      v = ei::to_f32<T>(q[(static_cast<size_t>(row0 + ppi) * nq + g * G + hhi) * D + d]) * scale;
+      v = ei::to_f32<T>(q[(static_cast<size_t>(row0 + ppi) * nq + g * G + hhi) * DQ + d]) * scale;
     Qs[idx] = v;
   }
 
   float m_r = kLowest, l_r = 0.f;
-  float acc[16];
+  float acc[kAcc];
 #pragma unroll
-  for (int k = 0; k < 16; ++k) acc[k] = 0.f;
+  for (int k = 0; k < kAcc; ++k) acc[k] = 0.f;
   const int nd = (DV + 15) / 16;
   const int nj = BC / 16;
 
@@ -88,22 +96,28 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
       const int phys = page_table[static_cast<size_t>(seq) * table_width + p];
       if (phys < 0) continue;  // a page the window has released: every key in it is masked
       const T* kp = k_pages + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
-      const T* vp = v_pages + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * DV;
+      const int DVS = values_in_keys ? D : DV;      // distance between two keys' values
+      const T* vp = values_in_keys
+                        ? kp
+                        : v_pages + (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * DV;
       for (int ch = 0; ch < chunks_per_page; ++ch) {
         const int key0 = p * EI_PAGE + ch * BC;
         if (key0 > hi_key) break;
         if (key0 + BC <= lo_key) continue;   // wholly before what any row of the item sees
         __syncthreads();
-        for (int idx = t; idx < BC * D; idx += kThreads) {
-          const int c = idx / D, d = idx % D;
+        for (int idx = t; idx < BC * DQ; idx += kThreads) {
+          const int c = idx / DQ, d = idx % DQ;
           const bool live = key0 + c <= hi_key;  // later slots hold stale bytes
-          const size_t off = static_cast<size_t>(ch * BC + c) * D + d;
-          Ks[c * (D + 1) + d] = live ? ei::to_f32<T>(kp[off]) : 0.f;
+          // with key_heads > 1 the piece d / D of the key lies in that kv head's page part
+          const T* src = KH > 1 ? k_pages + (static_cast<size_t>(phys) * nkv + d / D) * EI_PAGE * D
+                                : kp;
+          const size_t off = static_cast<size_t>(ch * BC + c) * D + (KH > 1 ? d % D : d);
+          Ks[c * (DQ + 1) + d] = live ? ei::to_f32<T>(src[off]) : 0.f;
         }
         for (int idx = t; idx < BC * DV; idx += kThreads) {
           const int c = idx / DV, d = idx % DV;
           const bool live = key0 + c <= hi_key;
-          const size_t off = static_cast<size_t>(ch * BC + c) * DV + d;
+          const size_t off = static_cast<size_t>(ch * BC + c) * DVS + d;
           Vs[c * DV + d] = live ? ei::to_f32<T>(vp[off]) : 0.f;
         }
         __syncthreads();
@@ -119,9 +133,9 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
                                  (chunk <= 0 || key / chunk == chunk_r);
             if (visible) {
               float dot = 0.f;
-              const float* qr = Qs + r * D;
-              const float* kr = Ks + c * (D + 1);
-              for (int d = 0; d < D; ++d) dot += qr[d] * kr[d];
+              const float* qr = Qs + r * DQ;
+              const float* kr = Ks + c * (DQ + 1);
+              for (int d = 0; d < DQ; ++d) dot += qr[d] * kr[d];
               dot -= slope * static_cast<float>(pos_r - key);
               s[j] = dot;
               row_max = fmaxf(row_max, dot);
@@ -149,7 +163,7 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
         __syncthreads();
         const float* pr = Ps + r * (BC + 1);
 #pragma unroll
-        for (int k = 0; k < 16; ++k) {
+        for (int k = 0; k < kAcc; ++k) {
           if (k < nd) {
             const int d = cc + 16 * k;
             float a = acc[k] * alpha;
@@ -170,20 +184,21 @@ attn_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
     const float alpha = expf(m_r - m_new);
     l_r = l_r * alpha + expf(sink - m_new);
 #pragma unroll
-    for (int k = 0; k < 16; ++k) acc[k] *= alpha;
+    for (int k = 0; k < kAcc; ++k) acc[k] *= alpha;
     m_r = m_new;
   }
   if (n_splits == 1) {
-    const float inv = l_r > 0.f ? 1.f / l_r : 0.f;
+    float inv = l_r > 0.f ? 1.f / l_r : 0.f;
+    if (gate) inv *= 1.0f / (1.0f + expf(-gate[static_cast<size_t>(row) * nq + head]));
     T* dst = out + (static_cast<size_t>(row) * nq + head) * DV;
 #pragma unroll
-    for (int k = 0; k < 16; ++k)
+    for (int k = 0; k < kAcc; ++k)
       if (k < nd && cc + 16 * k < DV) dst[cc + 16 * k] = ei::from_f32<T>(acc[k] * inv);
   } else {
     const size_t slot = (static_cast<size_t>(row) * nq + head) * n_splits + split;
     float* dst = part_o + slot * DV;
 #pragma unroll
-    for (int k = 0; k < 16; ++k)
+    for (int k = 0; k < kAcc; ++k)
       if (k < nd && cc + 16 * k < DV) dst[cc + 16 * k] = acc[k];
     if (cc == 0) {
       part_ml[slot * 2] = m_r;
@@ -197,7 +212,8 @@ template <typename T>
 __global__ void attn_merge_kernel(const float* __restrict__ part_o,
                                   const float* __restrict__ part_ml,
                                   const int32_t* __restrict__ row_seq, T* __restrict__ out, int nq,
-                                  int D, int n_splits, int total) {
+                                  int D, int n_splits, int total,
+                                  const float* __restrict__ gate) {
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
   const int lane = threadIdx.x % EI_WAVE;
   if (wave >= total) return;
@@ -208,7 +224,8 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o,
   for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
   float l = 0.f;
   for (int s = 0; s < n_splits; ++s) l += ml[2 * s + 1] * expf(ml[2 * s] - m);
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  float inv = l > 0.f ? 1.f / l : 0.f;
+  if (gate) inv *= 1.0f / (1.0f + expf(-gate[wave]));
   const float* po = part_o + static_cast<size_t>(wave) * n_splits * D;
   for (int d = lane; d < D; d += EI_WAVE) {
     float o = 0.f;
@@ -239,13 +256,19 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
                             const int32_t* row_seq, const int32_t* page_table, int table_width,
                             void* out, float* part_o, float* part_ml, int N, int nq, int nkv,
                             int D, int DV, int window, int chunk, const float* slopes,
-                            const float* sinks, float scale, int n_splits, hipStream_t stream) {
+                            const float* sinks, float scale, int n_splits, int key_heads,
+                            int values_in_keys, const float* gate, hipStream_t stream) {
   EI_REQUIRE(n_items > 0 && N > 0 && nq > 0 && nkv > 0, "attention: sizes must be positive");
   EI_REQUIRE(nq % nkv == 0, "attention: query heads must be a multiple of kv heads");
-  EI_REQUIRE(D >= 1 && D <= 256 && DV >= 1 && DV <= 256,
-             "attention: key and value head sizes must lie between 1 and 256");
+  EI_REQUIRE(key_heads == 1 || key_heads == nkv,
+             "attention: a query meets the keys of its own kv head or of all of them");
+  const int DQ = key_heads * D;
+  EI_REQUIRE(D >= 1 && DQ <= 1024 && DV >= 1 && DV <= 16 * kAcc,
+             "attention: keys of at most 1024 and values of at most 512 elements a head");
+  EI_REQUIRE(!values_in_keys || DV <= D, "attention: values inside keys cannot be wider than them");
+  EI_REQUIRE(values_in_keys || v_pages, "attention: null pointer");
   EI_REQUIRE(chunk >= 0, "attention: negative chunk");
-  EI_REQUIRE(q && k_pages && v_pages && out && item_seq && item_row0 && item_npos && row_pos &&
+  EI_REQUIRE(q && k_pages && out && item_seq && item_row0 && item_npos && row_pos &&
                  page_table && table_width > 0,
              "attention: null pointer");
   EI_REQUIRE(n_splits >= 1 && n_splits <= 64, "attention: splits must be between 1 and 64");
@@ -254,10 +277,25 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
   const int G = nq / nkv;
   const int Gb = G < kRows ? G : kRows;
   const int head_blocks = (G + Gb - 1) / Gb;
-  const int BC = chunk_keys(D > DV ? D : DV);
+  const int BC = chunk_keys(DQ > DV ? DQ : DV);
   const size_t lds =
-      sizeof(float) * (static_cast<size_t>(kRows) * D + static_cast<size_t>(BC) * (D + 1) +
+      sizeof(float) * (static_cast<size_t>(kRows) * DQ + static_cast<size_t>(BC) * (DQ + 1) +
                        static_cast<size_t>(BC) * DV + static_cast<size_t>(kRows) * (BC + 1));
+  if (lds > 64 * 1024) {      // beyond the default bound of a launch: ask for it, once
+    static bool raised = false;
+    if (!raised) {
+      const int most = 160 * 1024;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_generic_kernel<float>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
+          hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_generic_kernel<bf16_t>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess) {
+        (void)hipGetLastError();
+        EI_REQUIRE(false, "attention: the device refuses the LDS these head sizes need");
+      }
+      raised = true;
+    }
+  }
+  EI_REQUIRE(lds <= 160 * 1024, "attention: head sizes too large for the LDS");
   EI_REQUIRE(static_cast<long long>(nkv) * head_blocks <= 65535, "attention: too many heads");
   dim3 grid(n_items, nkv * head_blocks, n_splits);
   if (dtype == EI_F32) {
@@ -265,13 +303,13 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
         static_cast<const float*>(q), static_cast<const float*>(k_pages),
         static_cast<const float*>(v_pages), item_seq, item_row0, item_npos, row_pos, page_table,
         table_width, static_cast<float*>(out), part_o, part_ml, nq, nkv, D, DV, Gb, head_blocks,
-        BC, window, chunk, slopes, sinks, scale, n_splits);
+        BC, window, chunk, slopes, sinks, scale, n_splits, key_heads, values_in_keys, gate);
   } else if (dtype == EI_BF16) {
     attn_generic_kernel<bf16_t><<<grid, kThreads, lds, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
         static_cast<const bf16_t*>(v_pages), item_seq, item_row0, item_npos, row_pos, page_table,
         table_width, static_cast<bf16_t*>(out), part_o, part_ml, nq, nkv, D, DV, Gb, head_blocks,
-        BC, window, chunk, slopes, sinks, scale, n_splits);
+        BC, window, chunk, slopes, sinks, scale, n_splits, key_heads, values_in_keys, gate);
   } else {
     EI_REQUIRE(false, "attention: unknown dtype");
   }
@@ -286,10 +324,10 @@ extern "C" int ei_attention(const void* q, const void* k_pages, const void* v_pa
     const int blocks = (total * EI_WAVE + threads - 1) / threads;
     if (dtype == EI_F32)
       attn_merge_kernel<float><<<blocks, threads, 0, stream>>>(
-          part_o, part_ml, row_seq, static_cast<float*>(out), nq, DV, n_splits, total);
+          part_o, part_ml, row_seq, static_cast<float*>(out), nq, DV, n_splits, total, gate);
     else
       attn_merge_kernel<bf16_t><<<blocks, threads, 0, stream>>>(
-          part_o, part_ml, row_seq, static_cast<bf16_t*>(out), nq, DV, n_splits, total);
+          part_o, part_ml, row_seq, static_cast<bf16_t*>(out), nq, DV, n_splits, total, gate);
   }
   EI_LAUNCH_CHECK();
 }

@@ -24,11 +24,17 @@ PAGE_TOKENS = 64
 
 _SIGNATURES = {
     "rowwise": {
-        "ei_embed_gather": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ei_embed_gather": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float,
+                            c_void_p],
         "ei_add_rmsnorm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
                            c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int, c_int,
-                      c_void_p],
+                      c_int, c_void_p],
+        "ei_norm_add_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
+                             c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ei_concat_cast": [c_void_p, c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
+        "ei_set_rows": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_longlong, c_int,
+                        c_void_p],
         "ei_sum_slices": [c_void_p, c_int, c_longlong, c_void_p, c_longlong, c_void_p],
         "ei_bias_rows": [c_void_p, c_void_p, c_longlong, c_int, c_int, c_void_p],
         "ei_norm_add": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_float, c_void_p,
@@ -67,7 +73,30 @@ _SIGNATURES = {
         "ei_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
-                         c_int, c_void_p],
+                         c_int, c_int, c_int, c_void_p, c_void_p],
+    },
+    "head_ops": {
+        "ei_latent_down_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_float,
+                                 c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                 c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                 c_void_p],
+        "ei_head_matmul": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_int, c_int, c_void_p,
+                           c_int, c_void_p, c_int, c_longlong, c_int, c_int, c_int, c_int, c_int,
+                           c_int, c_void_p],
+        "ei_rotate_pairs": [c_void_p, c_int, c_int, c_longlong, c_longlong, c_int, c_int, c_void_p,
+                            c_void_p, c_void_p, c_int, c_longlong, c_int, c_int, c_int, c_int,
+                            c_int, c_void_p],
+        "ei_mix_heads": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                         c_void_p],
+    },
+    "mlstm": {
+        "ei_mlstm_state_floats": [c_int, c_int, c_int],
+        "ei_mlstm_proj_width": [c_int, c_int, c_int],
+        "ei_mlstm_walk": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p,
+                          c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                          c_int, c_int, c_int, c_float, c_float, c_float, c_void_p],
+        "ei_mlstm_out": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_float,
+                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "attention_mfma": {
         "ei_attn_decode_mfma_supported": [c_int, c_int],
@@ -223,7 +252,9 @@ def _splits(tensor: torch.Tensor, rows: int, width: int, name: str):
 
 
 # ---------------------------------------------------------------------------
-def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor,
+                 scale: float = 1.0) -> None:
+    """out[r] = table[ids[r]] * scale as float32."""
     lib = library("rowwise")
     n = ids.numel()
     vocab, hidden = table.shape
@@ -231,7 +262,7 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> N
         raise KernelError(f"embed_gather: out must be [{n}, {hidden}], got {list(out.shape)}")
     status = lib.ei_embed_gather(_gpu(ids, "ids", torch.int32), _gpu(table, "table"),
                                  _code(table, "table"), _gpu(out, "out", torch.float32), n,
-                                 hidden, vocab, _stream())
+                                 hidden, vocab, float(scale), _stream())
     _check(lib, status, "embed_gather")
 
 
@@ -263,15 +294,23 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     _check(lib, status, "add_rmsnorm")
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor, strip: int = 0) -> None:
-    """out = silu(gate) * up of [n, 2*inter] rows (or float32 slices of them).  strip = 0:
-    the gate columns come first, then the up columns; strip > 0: `strip` gate columns,
-    their `strip` up columns, and so on."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, strip: int = 0,
+           activation: str = "silu") -> None:
+    """out = act(gate) * up of [n, 2*inter] rows (or float32 slices of them), act "silu" or
+    "gelu_tanh".  strip = 0: the gate columns come first, then the up columns; strip > 0:
+    `strip` gate columns, their `strip` up columns, and so on."""
     lib = library("rowwise")
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"swiglu: unknown gate activation '{activation}'; "
+                          f"known: {sorted(GATE_ACTIVATIONS)}")
     n, inter = out.shape
     nsplit, stride = _splits(gate_up, n, 2 * inter, "gate_up")
     status = lib.ei_swiglu(_gpu(gate_up, "gate_up"), _code(gate_up, "gate_up"), nsplit, stride,
-                           _gpu(out, "out"), _code(out, "out"), n, inter, int(strip), _stream())
+                           _gpu(out, "out"), _code(out, "out"), n, inter, int(strip),
+                           GATE_ACTIVATIONS[activation], _stream())
     _check(lib, status, "swiglu")
 
 
@@ -314,6 +353,50 @@ def norm_add(residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, 
                              F32 if cast_out is None else _code(cast_out, "cast_out"), rows, hidden,
                              _stream())
     _check(lib, status, "norm_add")
+
+
+def norm_add_norm(residual: torch.Tensor, delta: torch.Tensor, w_after: torch.Tensor,
+                  w_next: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """residual [R, H] float32 += rmsnorm(sum of delta's slices) * w_after, then
+    out [R, H] = rmsnorm(residual) * w_next in out's type: one pass over the rows."""
+    lib = library("rowwise")
+    rows, hidden = residual.shape
+    nsplit, stride = _splits(delta, rows, hidden, "delta")
+    if w_after.numel() != hidden or w_next.numel() != hidden:
+        raise KernelError(f"norm_add_norm: weights must have {hidden} elements")
+    if tuple(out.shape) != (rows, hidden):
+        raise KernelError("norm_add_norm: out must have the residual's shape")
+    status = lib.ei_norm_add_norm(_gpu(residual, "residual", torch.float32), _gpu(delta, "delta"),
+                                  _code(delta, "delta"), nsplit, stride,
+                                  _gpu(w_after, "w_after", torch.float32),
+                                  _gpu(w_next, "w_next", torch.float32), float(eps),
+                                  _gpu(out, "out"), _code(out, "out"), rows, hidden, _stream())
+    _check(lib, status, "norm_add_norm")
+
+
+def concat_cast(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> None:
+    """out [R, 2H] = [a | b] for float32 a, b [R, H], in out's type."""
+    lib = library("rowwise")
+    rows, hidden = a.shape
+    if tuple(b.shape) != (rows, hidden) or tuple(out.shape) != (rows, 2 * hidden):
+        raise KernelError("concat_cast: a and b must be [rows, H] and out [rows, 2 H]")
+    status = lib.ei_concat_cast(_gpu(a, "a", torch.float32), _gpu(b, "b", torch.float32),
+                                _gpu(out, "out"), _code(out, "out"), rows, hidden, _stream())
+    _check(lib, status, "concat_cast")
+
+
+def set_rows(x: torch.Tensor, out: torch.Tensor, vector: Optional[torch.Tensor] = None) -> None:
+    """out [R, H] float32 = sum of x's slices (+ vector [H]): a product's result becomes the
+    float32 stream."""
+    lib = library("rowwise")
+    rows, hidden = out.shape
+    nsplit, stride = _splits(x, rows, hidden, "x")
+    if vector is not None and vector.numel() != hidden:
+        raise KernelError(f"set_rows: the vector must have {hidden} elements")
+    status = lib.ei_set_rows(_gpu(x, "x"), _code(x, "x"), nsplit, stride,
+                             None if vector is None else _gpu(vector, "vector", torch.float32),
+                             _gpu(out, "out", torch.float32), rows, hidden, _stream())
+    _check(lib, status, "set_rows")
 
 
 def cast_rows(source: torch.Tensor, out: torch.Tensor) -> None:
@@ -398,23 +481,40 @@ def attention_positions_per_item(group: int) -> int:
 def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos, row_seq,
               page_table, out, n_heads, n_kv_heads, head_dim, window=None, scale=None,
               n_splits=1, part_o=None, part_ml=None, value_dim=None, chunk=None, slopes=None,
-              sinks=None) -> None:
+              sinks=None, key_heads=1, values_in_keys=False, gate=None) -> None:
     """Generic causal attention over the paged cache (see attention_generic.hip).
     value_dim: head size of the values and of `out` (None: head_dim); chunk: a query sees only
     the keys of its own block of that many positions; slopes, sinks: float32 [n_heads], the
-    distance term's slope and the softmax's sink of every query head (None: none)."""
+    distance term's slope and the softmax's sink of every query head (None: none).
+    key_heads: 1, or n_kv_heads: a query row is then n_kv_heads * head_dim wide and meets the
+    keys of all kv heads of a position laid end to end (scores mixed over heads: see
+    `mix_heads`).  values_in_keys: the values are the first value_dim elements of the key
+    rows and `v_pages` is not read.  gate: float32 [rows, heads]; the output of a row and
+    head is multiplied by sigmoid(gate)."""
     lib = library("attention_generic")
     n = q.shape[0]
     value_dim = head_dim if value_dim is None else int(value_dim)
-    if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != (n, n_heads * value_dim):
-        raise KernelError("attention: q must be [rows, heads * head_dim] and out "
+    key_heads = int(key_heads)
+    if key_heads not in (1, n_kv_heads):
+        raise KernelError("attention: key_heads must be 1 or the number of kv heads")
+    if tuple(q.shape) != (n, n_heads * key_heads * head_dim) or \
+            tuple(out.shape) != (n, n_heads * value_dim):
+        raise KernelError("attention: q must be [rows, heads * key_heads * head_dim] and out "
                           "[rows, heads * value_dim]")
     expect = (n_kv_heads, PAGE_TOKENS, head_dim)
     expect_v = (k_pages.shape[0], n_kv_heads, PAGE_TOKENS, value_dim)
-    if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != expect_v:
-        raise KernelError(f"attention: pages must be [*, {expect}] and {list(expect_v)}")
+    if tuple(k_pages.shape[1:]) != expect:
+        raise KernelError(f"attention: key pages must be [*, {expect}]")
+    if values_in_keys:
+        if value_dim > head_dim:
+            raise KernelError("attention: values inside the keys cannot be wider than the keys")
+        v_pages = k_pages
+    elif tuple(v_pages.shape) != expect_v:
+        raise KernelError(f"attention: value pages must be {list(expect_v)}")
     if not (q.dtype == k_pages.dtype == v_pages.dtype == out.dtype):
         raise KernelError("attention: q, cache and out dtypes differ")
+    if gate is not None and (gate.dtype != torch.float32 or gate.numel() != n * n_heads):
+        raise KernelError("attention: the gate must be float32 [rows, heads]")
     if item_seq.numel() < n_items or item_row0.numel() < n_items or item_npos.numel() < n_items:
         raise KernelError("attention: work item arrays shorter than n_items")
     for name, per_head in (("slopes", slopes), ("sinks", sinks)):
@@ -438,8 +538,172 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
         n_kv_heads, head_dim, value_dim, int(window or 0), int(chunk or 0),
         None if slopes is None else _gpu(slopes, "slopes", torch.float32),
         None if sinks is None else _gpu(sinks, "sinks", torch.float32), float(scale), n_splits,
-        _stream())
+        key_heads, int(bool(values_in_keys)),
+        None if gate is None else _gpu(gate, "gate", torch.float32), _stream())
     _check(lib, status, "attention")
+
+
+# ---------------------------------------------------------------------------
+# per-head operations (head_ops.hip)
+def _rows_of(x, name):
+    """(rows, row width, nsplit, split stride) of [rows, width] or float32 slices of it."""
+    if x.dim() == 2:
+        return x.shape[0], x.shape[1], 1, 0
+    if x.dim() == 3 and x.dtype == torch.float32:
+        return x.shape[1], x.shape[2], x.shape[0], x.shape[1] * x.shape[2]
+    raise KernelError(f"{name} must be [rows, width] or float32 [slices, rows, width]")
+
+
+def latent_down_store(proj, q_norm_w, c_norm_w, eps, frequencies, row_pos, row_seq, page_table,
+                      q_latent, k_pages, gate_out, q_rank, kv_rank, rot_dim, n_gate,
+                      write_cache=True) -> None:
+    """One row of a fused down-projection [q_rank | kv_rank | rot_dim | n_gate]: the first two
+    parts are RMS-normed with their weights; the queries' latent goes to `q_latent` [rows,
+    q_rank], the keys' latent and the rotated last part (neighbouring pairs, angle position *
+    frequencies[i]) to the row's cache page `k_pages` [pages, 1, 64, kv_rank + rot_dim], the gate
+    logits to `gate_out` float32 [rows, n_gate]."""
+    lib = library("head_ops")
+    n, width, nsplit, stride = _rows_of(proj, "proj")
+    if width != q_rank + kv_rank + rot_dim + n_gate:
+        raise KernelError("latent_down_store: the projection's width does not fit its parts")
+    if tuple(q_latent.shape) != (n, q_rank):
+        raise KernelError("latent_down_store: q_latent must be [rows, q_rank]")
+    if q_norm_w.numel() != q_rank or c_norm_w.numel() != kv_rank:
+        raise KernelError("latent_down_store: norm weights must be as wide as the latents")
+    if rot_dim and (frequencies is None or frequencies.numel() != rot_dim // 2):
+        raise KernelError("latent_down_store: one frequency for every rotated pair")
+    if n_gate and (gate_out is None or gate_out.numel() < n * n_gate):
+        raise KernelError("latent_down_store: gate_out must be float32 [rows, n_gate]")
+    if row_pos.numel() < n or row_seq.numel() < n:
+        raise KernelError("latent_down_store: row metadata shorter than the rows")
+    if write_cache:
+        if tuple(k_pages.shape[1:]) != (1, PAGE_TOKENS, kv_rank + rot_dim):
+            raise KernelError("latent_down_store: pages must be [*, 1, 64, kv_rank + rot_dim]")
+        if k_pages.dtype != q_latent.dtype:
+            raise KernelError("latent_down_store: cache and q_latent dtypes differ")
+    status = lib.ei_latent_down_store(
+        _gpu(proj, "proj"), _code(proj, "proj"), nsplit, stride,
+        _gpu(q_norm_w, "q_norm_w", torch.float32), _gpu(c_norm_w, "c_norm_w", torch.float32),
+        float(eps), None if frequencies is None else _gpu(frequencies, "frequencies", torch.float32),
+        _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
+        _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
+        _gpu(q_latent, "q_latent"), _gpu(k_pages, "k_pages") if write_cache else None,
+        None if gate_out is None else _gpu(gate_out, "gate_out", torch.float32),
+        _code(q_latent, "q_latent"), n, q_rank, kv_rank, rot_dim, n_gate, int(write_cache),
+        _stream())
+    _check(lib, status, "latent_down_store")
+
+
+def head_matmul(x, matrices, y, heads, x_head, x_first, y_head, y_first) -> None:
+    """y[n, h * y_head + y_first + j] = sum_i x[n, h * x_head + x_first + i] * matrices[h, i, j]
+    for matrices [heads, K, J] of the storage type; x [rows, width] or float32 slices of it."""
+    lib = library("head_ops")
+    n, x_row, nsplit, stride = _rows_of(x, "x")
+    if matrices.dim() != 3 or matrices.shape[0] != heads:
+        raise KernelError("head_matmul: matrices must be [heads, K, J]")
+    if y.dim() != 2 or y.shape[0] != n:
+        raise KernelError("head_matmul: y must be [rows, width]")
+    _, k, j = matrices.shape
+    status = lib.ei_head_matmul(_gpu(x, "x"), _code(x, "x"), nsplit, stride, x_row, int(x_head),
+                                int(x_first), _gpu(matrices, "matrices"),
+                                _code(matrices, "matrices"), _gpu(y, "y"), _code(y, "y"),
+                                y.shape[1], int(y_head), int(y_first), n, heads, k, j, _stream())
+    _check(lib, status, "head_matmul")
+
+
+def rotate_pairs(x, frequencies, row_pos, y, heads, rot_dim, x_head, x_first, y_head,
+                 y_first) -> None:
+    """Elements (2i, 2i + 1) of x[n, h * x_head + x_first + 0..rot_dim] turn by the angle
+    row_pos[n] * frequencies[i] and go to y[n, h * y_head + y_first + ...]."""
+    lib = library("head_ops")
+    n, x_row, nsplit, stride = _rows_of(x, "x")
+    if y.dim() != 2 or y.shape[0] != n:
+        raise KernelError("rotate_pairs: y must be [rows, width]")
+    if frequencies.numel() != rot_dim // 2 or row_pos.numel() < n:
+        raise KernelError("rotate_pairs: one frequency a pair and one position a row")
+    status = lib.ei_rotate_pairs(_gpu(x, "x"), _code(x, "x"), nsplit, stride, x_row, int(x_head),
+                                 int(x_first), _gpu(frequencies, "frequencies", torch.float32),
+                                 _gpu(row_pos, "row_pos", torch.int32), _gpu(y, "y"),
+                                 _code(y, "y"), y.shape[1], int(y_head), int(y_first), n, heads,
+                                 int(rot_dim), _stream())
+    _check(lib, status, "rotate_pairs")
+
+
+def mix_heads(q, talk, out, heads, kv_heads, head_dim) -> None:
+    """out[n, h, c, :] = sum over the heads g of kv head c of talk[h, g] q[n, g, :]: with
+    `attention(..., key_heads=kv_heads)` the scores of these rows are the scores of q mixed
+    over heads by `talk` [heads, heads] (float32)."""
+    lib = library("head_ops")
+    n = q.shape[0]
+    if tuple(q.shape) != (n, heads * head_dim) or \
+            tuple(out.shape) != (n, heads * kv_heads * head_dim) or q.dtype != out.dtype:
+        raise KernelError("mix_heads: q must be [rows, heads * head_dim] and out "
+                          "[rows, heads * kv_heads * head_dim] of one type")
+    if talk.numel() != heads * heads:
+        raise KernelError("mix_heads: the mixing matrix must be [heads, heads]")
+    status = lib.ei_mix_heads(_gpu(q, "q"), _code(q, "q"), _gpu(talk, "talk", torch.float32),
+                              _gpu(out, "out"), n, heads, kv_heads, head_dim, _stream())
+    _check(lib, status, "mix_heads")
+
+
+# ---------------------------------------------------------------------------
+# matrix memory (mlstm.hip)
+def mlstm_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
+    """Floats of one sequence's state: per head S^T [value_dim, key_dim], n [key_dim], m."""
+    return heads * (value_dim * key_dim + key_dim + 1)
+
+
+def mlstm_proj_width(heads: int, key_dim: int, value_dim: int) -> int:
+    """Width of the fused projection [q | k | v | i | f | g]."""
+    return 2 * heads * key_dim + 2 * heads * value_dim + 2 * heads
+
+
+def mlstm_walk(proj, i_bias, f_bias, state, seq_in, seq_out, seq_count, seq_row0, o_raw, heads,
+               key_dim, value_dim, cap, q_scale, bottom_eps) -> None:
+    """The matrix memory's walk over the rows of a step (see mlstm.hip): proj [rows, width] or
+    float32 slices; state float32 [table rows, state floats]; o_raw float32 [rows, heads *
+    value_dim]."""
+    lib = library("mlstm")
+    n, width, nsplit, stride = _rows_of(proj, "proj")
+    if width != mlstm_proj_width(heads, key_dim, value_dim):
+        raise KernelError("mlstm_walk: the projection's width does not fit the shape")
+    if state.dim() != 2 or state.shape[1] < mlstm_state_floats(heads, key_dim, value_dim):
+        raise KernelError("mlstm_walk: state rows too short")
+    n_seqs = seq_count.numel()
+    if seq_in.numel() < n_seqs or seq_out.numel() < n_seqs or seq_row0.numel() < n_seqs:
+        raise KernelError("mlstm_walk: sequence metadata shorter than the sequences")
+    if tuple(o_raw.shape) != (n, heads * value_dim):
+        raise KernelError("mlstm_walk: o_raw must be [rows, heads * value_dim]")
+    if i_bias.numel() != heads or f_bias.numel() != heads:
+        raise KernelError("mlstm_walk: one gate bias a head")
+    status = lib.ei_mlstm_walk(
+        _gpu(proj, "proj"), _code(proj, "proj"), nsplit, stride,
+        _gpu(i_bias, "i_bias", torch.float32), _gpu(f_bias, "f_bias", torch.float32),
+        _gpu(state, "state", torch.float32), state.shape[1],
+        _gpu(seq_in, "seq_in", torch.int32), _gpu(seq_out, "seq_out", torch.int32),
+        _gpu(seq_count, "seq_count", torch.int32), _gpu(seq_row0, "seq_row0", torch.int32),
+        _gpu(o_raw, "o_raw", torch.float32), n_seqs, heads, key_dim, value_dim, float(cap),
+        float(q_scale), float(bottom_eps), _stream())
+    _check(lib, status, "mlstm_walk")
+
+
+def mlstm_out(o_raw, proj, norm_w, eps, row_seq, out, heads, key_dim, value_dim) -> None:
+    """out = rmsnorm per head (o_raw) * norm_w [heads * value_dim] * sigmoid(gate columns of
+    proj), in out's type."""
+    lib = library("mlstm")
+    n, width, nsplit, stride = _rows_of(proj, "proj")
+    if width != mlstm_proj_width(heads, key_dim, value_dim):
+        raise KernelError("mlstm_out: the projection's width does not fit the shape")
+    if tuple(o_raw.shape) != (n, heads * value_dim) or tuple(out.shape) != tuple(o_raw.shape):
+        raise KernelError("mlstm_out: o_raw and out must be [rows, heads * value_dim]")
+    if norm_w.numel() != heads * value_dim or row_seq.numel() < n:
+        raise KernelError("mlstm_out: the weight spans all heads; one sequence index a row")
+    status = lib.ei_mlstm_out(_gpu(o_raw, "o_raw", torch.float32), _gpu(proj, "proj"),
+                              _code(proj, "proj"), nsplit, stride,
+                              _gpu(norm_w, "norm_w", torch.float32), float(eps),
+                              _gpu(row_seq, "row_seq", torch.int32), _gpu(out, "out"),
+                              _code(out, "out"), n, heads, key_dim, value_dim, _stream())
+    _check(lib, status, "mlstm_out")
 
 
 def projection_norm_store(qkv, q_norm_w, k_norm_w, eps, row_pos, row_seq, page_table, q_out,

@@ -1,0 +1,278 @@
+// Matrix memory with exponential gates (the mLSTM cell): per head and sequence a state
+// S [key size, value size], a normaliser n [key size] and a running maximum m of the log gates,
+// all float32, carried from token to token.
+//
+// For token t with log input gate i_t and log forget gate f_t (m_0 = 0, S_0 = 0, n_0 = 0):
+//   m_t = max(f_t + m_{t-1}, i_t)
+//   S_t = e^(f_t + m_{t-1} - m_t) S_{t-1} + e^(i_t - m_t) k_t v_t^T     (n_t alike, with k_t alone)
+//   o_t = S_t^T q_t / (max(|n_t . q_t|, e^(-m_t)) + bottom_eps)
+// The gates come from two columns a head of the fused projection: with a cap c,
+//   i_t = c tanh((x_i + b_i) / c),   f_t = logsigmoid(c tanh((x_f + b_f) / c)).
+//
+// `mlstm_walk`: a block per (sequence, head, block of columns of S) walks the sequence's rows
+// of the step in order.  A thread owns 8 neighbouring rows of one column of S in registers (and
+// the same rows of n); the L = key size / 8 lanes of a column add their partial dot products
+// with wave shuffles.  Tokens come through LDS in tiles of 16: q, k, the block's columns of v,
+// and the three factors of every token, which one thread works out in order (the only chain
+// besides S itself).  The state is read from one row of the table and written, whole, to
+// another (the table has two versions a sequence).
+// `mlstm_out`: a wave a (row, head): RMS norm of the read-out, a weight as wide as all heads,
+// a sigmoid gate from the projection, one rounding.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kOwn = 8;        // rows of a column that a thread owns
+constexpr int kTile = 16;      // tokens in LDS at a time
+
+template <typename TI>
+__device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_stride) {
+  float x = 0.f;
+  for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TI>(p[s * split_stride]);
+  return x;
+}
+
+__device__ __forceinline__ float log_sigmoid(float z) {
+  return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+}
+
+// Column offsets of the fused projection [q | k | v | i | f | g].
+struct Columns {
+  int q, k, v, i, f, g, width;
+};
+
+__host__ __device__ inline Columns columns_of(int heads, int dim, int vdim) {
+  Columns c;
+  c.q = 0;
+  c.k = heads * dim;
+  c.v = 2 * heads * dim;
+  c.i = c.v + heads * vdim;
+  c.f = c.i + heads;
+  c.g = c.f + heads;
+  c.width = c.g + heads * vdim;
+  return c;
+}
+
+template <typename TI>
+__global__ void __launch_bounds__(kThreads)
+mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
+                  const float* __restrict__ i_bias, const float* __restrict__ f_bias,
+                  float* __restrict__ state, size_t state_stride,
+                  const int32_t* __restrict__ seq_in, const int32_t* __restrict__ seq_out,
+                  const int32_t* __restrict__ seq_count, const int32_t* __restrict__ seq_row0,
+                  float* __restrict__ o_raw, int heads, int dim, int vdim, int L, float cap,
+                  float q_scale, float bottom_eps) {
+  extern __shared__ float lds[];
+  const int dimP = L * kOwn;
+  const int CB = kThreads / L;                 // columns of S this block owns
+  float* qs = lds;                             // [kTile][dimP]
+  float* ks = qs + kTile * dimP;               // [kTile][dimP]
+  float* vs = ks + kTile * dimP;               // [kTile][CB]
+  float* keep_s = vs + kTile * CB;             // [kTile] e^(f + m' - m)
+  float* take_s = keep_s + kTile;              // [kTile] e^(i - m)
+  float* floor_s = take_s + kTile;             // [kTile] e^(-m)
+  float* gate_i = floor_s + kTile;             // [kTile] capped log input gate
+  float* gate_f = gate_i + kTile;              // [kTile] log forget gate
+
+  const int seq = blockIdx.x / heads, a = blockIdx.x % heads;
+  const int count = seq_count[seq];
+  if (count <= 0) return;                      // padding of a fixed-size batch
+  const int row0 = seq_row0[seq];
+  const Columns col_of = columns_of(heads, dim, vdim);
+  const int P = col_of.width;
+  const int t = threadIdx.x;
+  const int part = t % L, col_local = t / L;
+  const int col = blockIdx.y * CB + col_local;
+  const int r0 = part * kOwn;
+  const size_t head_floats = static_cast<size_t>(vdim) * dim + dim + 1;
+  const float* in = state + static_cast<size_t>(seq_in[seq]) * state_stride + a * head_floats;
+  float* out = state + static_cast<size_t>(seq_out[seq]) * state_stride + a * head_floats;
+
+  float S[kOwn], nn[kOwn];
+#pragma unroll
+  for (int r = 0; r < kOwn; ++r) {
+    const bool live = r0 + r < dim;
+    S[r] = (live && col < vdim) ? in[static_cast<size_t>(col) * dim + r0 + r] : 0.f;
+    nn[r] = live ? in[static_cast<size_t>(vdim) * dim + r0 + r] : 0.f;
+  }
+  float m_run = in[static_cast<size_t>(vdim) * dim + dim];      // used by thread 0 only
+
+  for (int t0 = 0; t0 < count; t0 += kTile) {
+    const int tn = min(kTile, count - t0);
+    __syncthreads();
+    for (int idx = t; idx < kTile * dimP; idx += kThreads) {
+      const int tt = idx / dimP, d = idx % dimP;
+      float qv = 0.f, kv = 0.f;
+      if (tt < tn && d < dim) {
+        const TI* src = proj + static_cast<size_t>(row0 + t0 + tt) * P + a * dim + d;
+        qv = sliced<TI>(src + col_of.q, nsplit, split_stride) * q_scale;
+        kv = sliced<TI>(src + col_of.k, nsplit, split_stride);
+      }
+      qs[idx] = qv;
+      ks[idx] = kv;
+    }
+    for (int idx = t; idx < kTile * CB; idx += kThreads) {
+      const int tt = idx / CB, c = blockIdx.y * CB + idx % CB;
+      float v = 0.f;
+      if (tt < tn && c < vdim)
+        v = sliced<TI>(proj + static_cast<size_t>(row0 + t0 + tt) * P + col_of.v + a * vdim + c,
+                       nsplit, split_stride);
+      vs[idx] = v;
+    }
+    if (t < tn) {
+      const TI* src = proj + static_cast<size_t>(row0 + t0 + t) * P;
+      const float xi = sliced<TI>(src + col_of.i + a, nsplit, split_stride) + i_bias[a];
+      const float xf = sliced<TI>(src + col_of.f + a, nsplit, split_stride) + f_bias[a];
+      gate_i[t] = cap * tanhf(xi / cap);
+      gate_f[t] = log_sigmoid(cap * tanhf(xf / cap));
+    }
+    __syncthreads();
+    if (t == 0) {
+      for (int tt = 0; tt < tn; ++tt) {
+        const float li = gate_i[tt], lf = gate_f[tt];
+        const float m_new = fmaxf(lf + m_run, li);
+        keep_s[tt] = expf(lf + m_run - m_new);
+        take_s[tt] = expf(li - m_new);
+        floor_s[tt] = expf(-m_new);
+        m_run = m_new;
+      }
+    }
+    __syncthreads();
+    for (int tt = 0; tt < tn; ++tt) {
+      const float keep = keep_s[tt], take = take_s[tt];
+      const float tv = take * vs[tt * CB + col_local];
+      const float* kr = ks + tt * dimP + r0;
+      const float* qr = qs + tt * dimP + r0;
+      float dot_s = 0.f, dot_n = 0.f;
+#pragma unroll
+      for (int r = 0; r < kOwn; ++r) {
+        const float k = kr[r], q = qr[r];
+        S[r] = keep * S[r] + k * tv;
+        nn[r] = keep * nn[r] + take * k;
+        dot_s += S[r] * q;
+        dot_n += nn[r] * q;
+      }
+      for (int offset = L / 2; offset > 0; offset >>= 1) {
+        dot_s += __shfl_xor(dot_s, offset, EI_WAVE);
+        dot_n += __shfl_xor(dot_n, offset, EI_WAVE);
+      }
+      if (part == 0 && col < vdim)
+        o_raw[static_cast<size_t>(row0 + t0 + tt) * heads * vdim + a * vdim + col] =
+            dot_s / (fmaxf(fabsf(dot_n), floor_s[tt]) + bottom_eps);
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < kOwn; ++r) {
+    if (r0 + r < dim) {
+      if (col < vdim) out[static_cast<size_t>(col) * dim + r0 + r] = S[r];
+      if (blockIdx.y == 0 && col_local == 0) out[static_cast<size_t>(vdim) * dim + r0 + r] = nn[r];
+    }
+  }
+  if (blockIdx.y == 0 && t == 0) out[static_cast<size_t>(vdim) * dim + dim] = m_run;
+}
+
+// One wave per (row, head).
+template <typename TI, typename TO>
+__global__ void mlstm_out_kernel(const float* __restrict__ o_raw, const TI* __restrict__ proj,
+                                 int nsplit, size_t split_stride,
+                                 const float* __restrict__ norm_w, float eps,
+                                 const int32_t* __restrict__ row_seq, TO* __restrict__ out,
+                                 int heads, int dim, int vdim, int total) {
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
+  const int lane = threadIdx.x % EI_WAVE;
+  if (wave >= total) return;
+  const int row = wave / heads, a = wave % heads;
+  if (row_seq[row] < 0) return;
+  const Columns col_of = columns_of(heads, dim, vdim);
+  const float* o = o_raw + (static_cast<size_t>(row) * heads + a) * vdim;
+  float sum = 0.f;
+  for (int j = lane; j < vdim; j += EI_WAVE) sum += o[j] * o[j];
+  sum = ei::wave_sum(sum);
+  const float inv = 1.0f / sqrtf(sum / static_cast<float>(vdim) + eps);
+  const TI* g = proj + static_cast<size_t>(row) * col_of.width + col_of.g + a * vdim;
+  for (int j = lane; j < vdim; j += EI_WAVE) {
+    const float gate = 1.0f / (1.0f + expf(-sliced<TI>(g + j, nsplit, split_stride)));
+    out[(static_cast<size_t>(row) * heads + a) * vdim + j] =
+        ei::from_f32<TO>((o[j] * inv) * norm_w[a * vdim + j] * gate);
+  }
+}
+
+int lanes_for(int dim) {
+  int L = 1;
+  while (L * kOwn < dim) L *= 2;
+  return L;
+}
+
+}  // namespace
+
+// Floats of one sequence's state: per head S^T [vdim, dim], n [dim], m.
+extern "C" int ei_mlstm_state_floats(int heads, int dim, int vdim) {
+  return heads * (vdim * dim + dim + 1);
+}
+
+// Width of the fused projection [q | k | v | i | f | g].
+extern "C" int ei_mlstm_proj_width(int heads, int dim, int vdim) {
+  return columns_of(heads, dim, vdim).width;
+}
+
+// proj: [nsplit][N, width]; state: rows of `state_stride` floats; seq_in / seq_out: the row
+// each sequence's state is read from and written to; o_raw: float32 [N, heads * vdim].
+extern "C" int ei_mlstm_walk(const void* proj, int dtype, int nsplit, long long split_stride,
+                             const float* i_bias, const float* f_bias, float* state,
+                             long long state_stride, const int32_t* seq_in, const int32_t* seq_out,
+                             const int32_t* seq_count, const int32_t* seq_row0, float* o_raw,
+                             int n_seqs, int heads, int dim, int vdim, float cap, float q_scale,
+                             float bottom_eps, hipStream_t stream) {
+  EI_REQUIRE(n_seqs > 0 && heads > 0 && vdim > 0 && nsplit >= 1, "mlstm_walk: bad sizes");
+  EI_REQUIRE(dim >= 1 && dim <= 256, "mlstm_walk: the key size must lie in 1..256");
+  EI_REQUIRE(cap > 0.f, "mlstm_walk: the cap of the gates must be positive");
+  EI_REQUIRE(proj && i_bias && f_bias && state && seq_in && seq_out && seq_count && seq_row0 &&
+                 o_raw,
+             "mlstm_walk: null pointer");
+  EI_REQUIRE(state_stride >= ei_mlstm_state_floats(heads, dim, vdim),
+             "mlstm_walk: state rows too short");
+  const int L = lanes_for(dim);
+  const int CB = kThreads / L;
+  const size_t lds = sizeof(float) * (2 * static_cast<size_t>(kTile) * L * kOwn +
+                                      static_cast<size_t>(kTile) * CB + 5 * kTile);
+  EI_REQUIRE(static_cast<long long>(n_seqs) * heads <= 0x7fffffffLL, "mlstm_walk: too many blocks");
+  dim3 grid(n_seqs * heads, (vdim + CB - 1) / CB);
+  const size_t ss = static_cast<size_t>(split_stride);
+  if (dtype == EI_F32)
+    mlstm_walk_kernel<float><<<grid, kThreads, lds, stream>>>(
+        static_cast<const float*>(proj), nsplit, ss, i_bias, f_bias, state,
+        static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, heads, dim,
+        vdim, L, cap, q_scale, bottom_eps);
+  else if (dtype == EI_BF16)
+    mlstm_walk_kernel<bf16_t><<<grid, kThreads, lds, stream>>>(
+        static_cast<const bf16_t*>(proj), nsplit, ss, i_bias, f_bias, state,
+        static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, heads, dim,
+        vdim, L, cap, q_scale, bottom_eps);
+  else
+    EI_REQUIRE(false, "mlstm_walk: unknown dtype");
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_mlstm_out(const float* o_raw, const void* proj, int in_dtype, int nsplit,
+                            long long split_stride, const float* norm_w, float eps,
+                            const int32_t* row_seq, void* out, int out_dtype, int N, int heads,
+                            int dim, int vdim, hipStream_t stream) {
+  EI_REQUIRE(N > 0 && heads > 0 && dim > 0 && vdim > 0 && nsplit >= 1, "mlstm_out: bad sizes");
+  EI_REQUIRE(o_raw && proj && norm_w && row_seq && out, "mlstm_out: null pointer");
+  const int total = N * heads;
+  const int threads = 256;
+  const int blocks = (total * EI_WAVE + threads - 1) / threads;
+  const size_t ss = static_cast<size_t>(split_stride);
+#define EI_MO_CASE(TI, TO)                                                                   \
+  mlstm_out_kernel<TI, TO><<<blocks, threads, 0, stream>>>(                                  \
+      o_raw, static_cast<const TI*>(proj), nsplit, ss, norm_w, eps, row_seq,                 \
+      static_cast<TO*>(out), heads, dim, vdim, total)
+  if (in_dtype == EI_F32 && out_dtype == EI_F32) EI_MO_CASE(float, float);
+  else if (in_dtype == EI_F32 && out_dtype == EI_BF16) EI_MO_CASE(float, bf16_t);
+  else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_MO_CASE(bf16_t, bf16_t);
+  else EI_REQUIRE(false, "mlstm_out: unsupported dtype combination");
+#undef EI_MO_CASE
+  EI_LAUNCH_CHECK();
+}

@@ -12,7 +12,7 @@ namespace {
 
 template <typename T>
 __global__ void embed_gather_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
-                                    float* __restrict__ out, int H, int V) {
+                                    float* __restrict__ out, int H, int V, float scale) {
   const int row = blockIdx.x;
   const int id = ids[row];
   float* dst = out + static_cast<size_t>(row) * H;
@@ -21,7 +21,7 @@ __global__ void embed_gather_kernel(const int32_t* __restrict__ ids, const T* __
     return;
   }
   const T* src = table + static_cast<size_t>(id) * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ei::to_f32<T>(src[i]);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ei::to_f32<T>(src[i]) * scale;
 }
 
 // One block per output row.  x = residual[src] (+ sum over splits of delta[s][src]);
@@ -137,13 +137,19 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* _
 
 // Where gate and up of output column `col` lie in a row of 2I: the halves [gate | up]
 // (strip = 0), or strips of `strip` gate columns followed by their `strip` up columns.
+// gate activations of the C interface: 0 silu, 1 the tanh form of gelu
+template <typename TO> __device__ __forceinline__ float gate_act(float x, int act) {
+  if (act == 0) return ei::silu<TO>(x);
+  return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+
 __device__ __forceinline__ size_t gate_column(size_t col, int strip) {
   return strip ? (col / strip) * 2 * strip + col % strip : col;
 }
 
 template <typename TI, typename TO>
 __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
-                              TO* __restrict__ out, int I, size_t total, int strip) {
+                              TO* __restrict__ out, int I, size_t total, int strip, int act) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   const size_t up_offset = strip ? strip : I;
@@ -155,7 +161,7 @@ __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t
       gate += ei::to_f32<TI>(g[s * split_stride]);
       up += ei::to_f32<TI>(g[s * split_stride + up_offset]);
     }
-    out[idx] = ei::from_f32<TO>(ei::silu<TO>(gate) * up);
+    out[idx] = ei::from_f32<TO>(gate_act<TO>(gate, act) * up);
   }
 }
 
@@ -163,7 +169,7 @@ __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t
 // 16-byte (bfloat16) or 2 x 16-byte (float32) accesses.
 template <typename TI, typename TO>
 __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
-                                  TO* __restrict__ out, int I, size_t total_octets, int strip) {
+                                  TO* __restrict__ out, int I, size_t total_octets, int strip, int act) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   const int octets_per_row = I / 8;
@@ -201,8 +207,8 @@ __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, si
     float y0[4], y1[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      y0[i] = ei::silu<TO>(gate[i]) * up[i];
-      y1[i] = ei::silu<TO>(gate[i + 4]) * up[i + 4];
+      y0[i] = gate_act<TO>(gate[i], act) * up[i];
+      y1[i] = gate_act<TO>(gate[i + 4], act) * up[i + 4];
     }
     TO* dst = out + row * I + col;
     Vec4<TO>::store(dst, y0);
@@ -262,16 +268,16 @@ extern "C" int ei_sum_slices(const float* in, int nsplit, long long stride, floa
 }
 
 extern "C" int ei_embed_gather(const int32_t* ids, const void* table, int table_dtype, float* out,
-                               int N, int H, int V, hipStream_t stream) {
+                               int N, int H, int V, float scale, hipStream_t stream) {
   EI_REQUIRE(N > 0 && H > 0 && V > 0, "embed_gather: sizes must be positive");
   EI_REQUIRE(ids && table && out, "embed_gather: null pointer");
   const int threads = H >= 1024 ? 256 : 64;
   if (table_dtype == EI_F32)
     embed_gather_kernel<float><<<N, threads, 0, stream>>>(ids, static_cast<const float*>(table),
-                                                          out, H, V);
+                                                          out, H, V, scale);
   else if (table_dtype == EI_BF16)
     embed_gather_kernel<bf16_t><<<N, threads, 0, stream>>>(ids, static_cast<const bf16_t*>(table),
-                                                           out, H, V);
+                                                           out, H, V, scale);
   else
     EI_REQUIRE(false, "embed_gather: unknown table dtype");
   EI_LAUNCH_CHECK();
@@ -348,8 +354,10 @@ extern "C" int ei_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
 // gate_up: [nsplit][N, 2I], out: [N, I].  strip = 0: gate columns first, then up columns;
 // strip > 0 (a divisor of I): `strip` gate columns, their `strip` up columns, and so on.
 extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long long split_stride,
-                         void* out, int out_dtype, int N, int I, int strip, hipStream_t stream) {
+                         void* out, int out_dtype, int N, int I, int strip, int act,
+                         hipStream_t stream) {
   EI_REQUIRE(N > 0 && I > 0 && nsplit >= 1, "swiglu: sizes must be positive");
+  EI_REQUIRE(act == 0 || act == 1, "swiglu: unknown gate activation");
   EI_REQUIRE(gate_up && out, "swiglu: null pointer");
   EI_REQUIRE(strip >= 0 && (strip == 0 || I % strip == 0), "swiglu: the strip must divide the width");
   const size_t total = static_cast<size_t>(N) * I;
@@ -361,13 +369,13 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
     if (vblocks > ei_compute_units() * 32) vblocks = ei_compute_units() * 32;
     if (in_dtype == EI_F32 && out_dtype == EI_F32)
       swiglu_vec_kernel<float, float><<<vblocks, threads, 0, stream>>>(
-          static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets, strip);
+          static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets, strip, act);
     else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
       swiglu_vec_kernel<float, bf16_t><<<vblocks, threads, 0, stream>>>(
-          static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip);
+          static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act);
     else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
       swiglu_vec_kernel<bf16_t, bf16_t><<<vblocks, threads, 0, stream>>>(
-          static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip);
+          static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act);
     else
       EI_REQUIRE(false, "swiglu: unsupported dtype combination");
     EI_LAUNCH_CHECK();
@@ -376,13 +384,13 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
   if (blocks > ei_compute_units() * 32) blocks = ei_compute_units() * 32;
   if (in_dtype == EI_F32 && out_dtype == EI_F32)
     swiglu_kernel<float, float><<<blocks, threads, 0, stream>>>(
-        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total, strip);
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total, strip, act);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
     swiglu_kernel<float, bf16_t><<<blocks, threads, 0, stream>>>(
-        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip);
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act);
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
     swiglu_kernel<bf16_t, bf16_t><<<blocks, threads, 0, stream>>>(
-        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip);
+        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act);
   else
     EI_REQUIRE(false, "swiglu: unsupported dtype combination");
   EI_LAUNCH_CHECK();
@@ -639,5 +647,137 @@ extern "C" int ei_activation(const void* in, int in_dtype, int nsplit, long long
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16) EI_ACT(bf16_t, bf16_t);
   else EI_REQUIRE(false, "activation: unsupported dtype combination");
 #undef EI_ACT
+  EI_LAUNCH_CHECK();
+}
+
+
+// ---------------------------------------------------------------------------------------
+// Kernels for blocks with a norm on both sides of every sublayer, and for a stream that is
+// made anew from two streams.
+namespace {
+
+// One block per row.  x = sum over slices of delta[row]; y = residual[row] + x * rsqrt(mean(x^2)
+// + eps) * w_after (stored back); out[row] = y * rsqrt(mean(y^2) + eps) * w_next in the storage
+// type: the norm on a sublayer's output, the addition and the next sublayer's input norm in
+// one pass over the row.
+template <typename TD, typename TO>
+__global__ void norm_add_norm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                     int nsplit, size_t split_stride,
+                                     const float* __restrict__ w_after,
+                                     const float* __restrict__ w_next, float eps,
+                                     TO* __restrict__ out, int H) {
+  extern __shared__ float row_values[];
+  __shared__ float scratch[16];
+  const size_t base = static_cast<size_t>(blockIdx.x) * H;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const TD* d = delta + base + i;
+    float x = 0.f;
+    for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TD>(d[s * split_stride]);
+    row_values[i] = x;
+    sum += x * x;
+  }
+  const float inv = 1.0f / sqrtf(ei::block_sum(sum, scratch) / static_cast<float>(H) + eps);
+  float sum2 = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float y = residual[base + i] + (row_values[i] * inv) * w_after[i];
+    residual[base + i] = y;
+    row_values[i] = y;
+    sum2 += y * y;
+  }
+  const float inv2 = 1.0f / sqrtf(ei::block_sum(sum2, scratch) / static_cast<float>(H) + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    out[base + i] = ei::from_f32<TO>((row_values[i] * inv2) * w_next[i]);
+}
+
+// out[r] = [a[r] | b[r]] in the storage type: two float32 streams side by side as the operand
+// of one product.
+template <typename TO>
+__global__ void concat_cast_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                   TO* __restrict__ out, int H, size_t n) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = start; i < n; i += step) {
+    const size_t row = i / (2 * H);
+    const int col = static_cast<int>(i % (2 * H));
+    const float v = col < H ? a[row * H + col] : b[row * H + col - H];
+    out[i] = ei::from_f32<TO>(v);
+  }
+}
+
+// out[r, j] = sum over slices of x[s][r, j] + vec[j]: a product's result takes the place of
+// the float32 stream.
+template <typename TD>
+__global__ void set_rows_kernel(const TD* __restrict__ x, int nsplit, size_t split_stride,
+                                const float* __restrict__ vec, float* __restrict__ out, int H,
+                                size_t n) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = start; i < n; i += step) {
+    float total = 0.f;
+    for (int s = 0; s < nsplit; ++s) total += ei::to_f32<TD>(x[s * split_stride + i]);
+    out[i] = vec ? total + vec[i % H] : total;
+  }
+}
+
+}  // namespace
+
+extern "C" int ei_norm_add_norm(float* residual, const void* delta, int delta_dtype, int nsplit,
+                                long long split_stride, const float* w_after, const float* w_next,
+                                float eps, void* out, int out_dtype, int N, int H,
+                                hipStream_t stream) {
+  EI_REQUIRE(N > 0 && H > 0 && nsplit >= 1, "norm_add_norm: sizes must be positive");
+  EI_REQUIRE(residual && delta && w_after && w_next && out, "norm_add_norm: null pointer");
+  EI_REQUIRE(static_cast<size_t>(H) * sizeof(float) <= 60 * 1024, "norm_add_norm: row too wide");
+  const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 128);
+  const size_t lds = static_cast<size_t>(H) * sizeof(float);
+  const size_t ss = static_cast<size_t>(split_stride);
+#define EI_NAN_CASE(TD, TO)                                                                  \
+  norm_add_norm_kernel<TD, TO><<<N, threads, lds, stream>>>(                                 \
+      residual, static_cast<const TD*>(delta), nsplit, ss, w_after, w_next, eps,             \
+      static_cast<TO*>(out), H)
+  if (delta_dtype == EI_F32 && out_dtype == EI_F32) EI_NAN_CASE(float, float);
+  else if (delta_dtype == EI_F32 && out_dtype == EI_BF16) EI_NAN_CASE(float, bf16_t);
+  else if (delta_dtype == EI_BF16 && out_dtype == EI_BF16) EI_NAN_CASE(bf16_t, bf16_t);
+  else EI_REQUIRE(false, "norm_add_norm: unsupported dtype combination");
+#undef EI_NAN_CASE
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_concat_cast(const float* a, const float* b, void* out, int out_dtype,
+                              long long rows, int H, hipStream_t stream) {
+  EI_REQUIRE(a && b && out && rows > 0 && H > 0, "concat_cast: bad arguments");
+  const size_t n = static_cast<size_t>(rows) * 2 * H;
+  const int threads = 256;
+  size_t blocks = (n + threads - 1) / threads;
+  if (blocks > ei_compute_units() * 16) blocks = ei_compute_units() * 16;
+  if (out_dtype == EI_F32)
+    concat_cast_kernel<float><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+        a, b, static_cast<float*>(out), H, n);
+  else if (out_dtype == EI_BF16)
+    concat_cast_kernel<bf16_t><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+        a, b, static_cast<bf16_t*>(out), H, n);
+  else
+    EI_REQUIRE(false, "concat_cast: unknown dtype");
+  EI_LAUNCH_CHECK();
+}
+
+extern "C" int ei_set_rows(const void* x, int x_dtype, int nsplit, long long split_stride,
+                           const float* vec, float* out, long long rows, int H,
+                           hipStream_t stream) {
+  EI_REQUIRE(x && out && rows > 0 && H > 0 && nsplit >= 1, "set_rows: bad arguments");
+  const size_t n = static_cast<size_t>(rows) * H;
+  const int threads = 256;
+  size_t blocks = (n + threads - 1) / threads;
+  if (blocks > ei_compute_units() * 16) blocks = ei_compute_units() * 16;
+  const size_t ss = static_cast<size_t>(split_stride);
+  if (x_dtype == EI_F32)
+    set_rows_kernel<float><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+        static_cast<const float*>(x), nsplit, ss, vec, out, H, n);
+  else if (x_dtype == EI_BF16)
+    set_rows_kernel<bf16_t><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+        static_cast<const bf16_t*>(x), nsplit, ss, vec, out, H, n);
+  else
+    EI_REQUIRE(false, "set_rows: unknown dtype");
   EI_LAUNCH_CHECK();
 }

@@ -18,8 +18,11 @@ replace in a subclass that it registers as its `model_factory`, keeping the rest
   final_hidden(ctx, residual, pending) -> h   [wanted rows, hidden] in the storage type
   logits(ctx, h) -> float32 [wanted rows, vocab]
 
-(a scaled embedding overrides `embed`, a cap on the logits `logits`, a model without a
-final norm `final_hidden`).  A subclass whose methods launch anything that a HIP graph
+(a cap on the logits overrides `logits`, a model without a final norm `final_hidden`).  Two
+variations are options of the spec and need no subclass: `embedding_scale` multiplies the
+embedding rows, and `loop` (`config.specs.LoopSpec`) runs a span of layers several times, each
+pass with caches of its own, the stream being made anew before every pass from itself and the
+embedding output by a matrix [hidden, 2 hidden] and a vector per pass.  A subclass whose methods launch anything that a HIP graph
 cannot hold says so with `seams_capture_safe = False`; decode then runs eagerly.
 """
 from __future__ import annotations
@@ -28,7 +31,7 @@ from typing import Callable, Dict, Mapping, Tuple
 
 import torch
 
-from ..config.specs import ModelSpec
+from ..config.specs import ModelSpec, pass_starts
 from ..csrc import lib
 from ..parts.linear import Linear
 from ..parts.registry import lookup
@@ -57,6 +60,10 @@ def model_parameters(spec: ModelSpec) -> Dict[str, ParamSpec]:
         params[f"final_norm.{name}"] = param
     params["head.weight"] = ParamSpec((spec.vocab_size, spec.hidden_size))
     params["head.bias"] = ParamSpec((spec.vocab_size,), optional=True)
+    if spec.loop is not None:
+        params["loop.in.weight"] = ParamSpec((spec.hidden_size, 2 * spec.hidden_size),
+                                             scale=(2.0 * spec.hidden_size) ** -0.5)
+        params["loop.step"] = ParamSpec((spec.loop.times, spec.hidden_size), scale=0.1)
     return params
 
 
@@ -148,6 +155,14 @@ class DecoderModel:
                                bias=params.get("head.bias"))
         else:  # tied: the head is the embedding table itself (no copy: same type and device)
             self.head = Linear(self.embed, self.dtype, self.device, bias=params.get("head.bias"))
+        self.loop_in = self.loop_step = None
+        self._pass_starts = {}
+        if spec.loop is not None:
+            self.loop_in = Linear(params["loop.in.weight"], self.dtype, self.device)
+            self.loop_step = params["loop.step"].to(device=self.device,
+                                                    dtype=torch.float32).contiguous()
+            self._pass_starts = {run: turn for turn, run in
+                                 enumerate(pass_starts(len(spec.layers), spec.loop))}
 
     @staticmethod
     def kernel_libraries(spec: ModelSpec, dtype):
@@ -213,6 +228,8 @@ class DecoderModel:
         if not self.seams_capture_safe:
             return False
         parts = [self.final_norm, self.head]
+        if self.loop_in is not None:
+            parts.append(self.loop_in)
         for layer in self.layers:
             parts += [layer, *members_of(layer)]
         return all(bool(getattr(part, "capture_safe", False)) for part in parts)
@@ -220,6 +237,8 @@ class DecoderModel:
     def capture_rows(self) -> int:
         """Most rows of a step for which `capture_safe` holds: the least any part allows."""
         rows = self.head.capture_rows
+        if self.loop_in is not None:
+            rows = min(rows, self.loop_in.capture_rows)
         for layer in self.layers:
             for part in (layer, *members_of(layer)):
                 rows = min(rows, getattr(part, "capture_rows", 1 << 30))
@@ -242,6 +261,8 @@ class DecoderModel:
             visit(layer)
         visit(self.final_norm)
         visit(self.head)
+        visit(self.loop_in)
+        visit(self.loop_step)
         return total
 
     # ------------------------------------------------------------------
@@ -276,16 +297,40 @@ class DecoderModel:
         """The rows of the embedding table that the step's tokens name, as the float32
         residual stream [rows, hidden]."""
         residual = ctx.buffer("residual", (ctx.n_rows, self.spec.hidden_size), torch.float32)
-        lib.embed_gather(ctx.meta.tokens, self.embed, residual)
+        lib.embed_gather(ctx.meta.tokens, self.embed, residual, self.spec.embedding_scale)
         return residual
 
     def run_layers(self, ctx, residual):
         """The layers in the order of the schedule.  Returns the last delta, which is not
         added to the residual yet (the norm that follows adds it while it reads the row)."""
         pending = None
-        for entry in self.spec.schedule:
+        embedded = None
+        if self.loop_in is not None:
+            # the embedding output, which every pass of the loop reads again
+            # (gathered a second time: the layers before the loop have changed the stream)
+            embedded = ctx.buffer("loop.x0", tuple(residual.shape), torch.float32)
+            lib.embed_gather(ctx.meta.tokens, self.embed, embedded, self.spec.embedding_scale)
+        for run, entry in enumerate(self.spec.schedule):
+            turn = self._pass_starts.get(run)
+            if turn is not None:
+                pending = self.enter_pass(ctx, residual, pending, embedded, turn)
             pending = self.layers[entry.layer].forward(ctx, residual, pending, entry)
         return pending
+
+    def enter_pass(self, ctx, residual, pending, embedded, turn: int):
+        """Before pass `turn` of the loop: x <- W [x ; x0] + step[turn], with x0 the embedding
+        output.  The product reads both streams in the step's storage type; its float32 result
+        takes the stream's place."""
+        if pending is not None:
+            raise ValueError("a pass of the loop starts after a block that left a delta pending")
+        rows, hidden = residual.shape
+        both = ctx.buffer("loop.both", (rows, 2 * hidden))
+        lib.concat_cast(residual, embedded, both)
+        made = self.loop_in.forward(ctx, both, "loop.made")
+        ctx.release(both)
+        lib.set_rows(made, residual, self.loop_step[turn])
+        ctx.release(made)
+        return None
 
     def final_hidden(self, ctx, residual, pending) -> torch.Tensor:
         """The normalised rows that the head reads: only the wanted ones."""

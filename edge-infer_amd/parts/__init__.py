@@ -1,25 +1,31 @@
 from .attention import Attention
 from .base import KVRequest, StateRequest, StepContext, Workspace
-from .block import OutputNormBlock, PreNormBlock
+from .block import OutputNormBlock, PreNormBlock, SandwichBlock
 from .delta import GatedDelta
+from .latent import LatentAttention
 from .linear import Linear
 from .mlp import DenseMLP, GatedMLP
+from .mlstm import MatrixMemory
 from .norm import RMSNorm
 from .registry import (lookup, register_block, register_feed_forward, register_mixer,
                        register_norm, register_position, unregister)
-from .rope import NoPosition, RotaryTable
+from .rope import NoPosition, RotaryFrequencies, RotaryTable
 
 register_mixer("attention", Attention)
 register_mixer("gated_delta", GatedDelta)
+register_mixer("latent_attention", LatentAttention)
+register_mixer("mlstm", MatrixMemory)
 register_feed_forward("gated_mlp", GatedMLP)
 register_feed_forward("dense_mlp", DenseMLP)
 register_norm("rmsnorm", RMSNorm)
 register_position("rope", RotaryTable)
 register_position("none", NoPosition)
+register_position("rope_pairs", RotaryFrequencies)
 register_block("prenorm", PreNormBlock)
 register_block("outnorm", OutputNormBlock)
+register_block("sandwich", SandwichBlock)
 
 __all__ = ["Attention", "KVRequest", "StateRequest", "StepContext", "Workspace", "PreNormBlock",
-           "OutputNormBlock", "GatedDelta", "DenseMLP", "Linear", "GatedMLP", "RMSNorm", "lookup", "register_block", "register_feed_forward",
+           "OutputNormBlock", "SandwichBlock", "GatedDelta", "LatentAttention", "MatrixMemory", "RotaryFrequencies", "DenseMLP", "Linear", "GatedMLP", "RMSNorm", "lookup", "register_block", "register_feed_forward",
            "register_mixer", "register_norm", "register_position", "unregister", "NoPosition",
            "RotaryTable"]

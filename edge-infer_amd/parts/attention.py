@@ -14,7 +14,13 @@ float32-arithmetic kernels): values narrower or wider than keys (`value_dim`), o
 over the whole q and the whole k projection instead of one per head (`qk_norm_scope =
 "projection"`), visibility in blocks of `chunk` positions counted from the sequence's start,
 a distance term slope_h (i - j) taken off the score with slope_h = 2^(-r (h + 1) / heads)
-(`distance_slope_range` = r), and a learned `sink` per head in the softmax's denominator.
+(`distance_slope_range` = r), a learned `sink` per head in the softmax's denominator or a
+plain 1 there (`unit_sink`), and `talking_heads`: a learned matrix T [heads, heads] mixes the
+scaled scores of every (query, key) pair over the heads before the softmax.  A mix of scores is
+the score of mixed queries: with the heads g of kv head c sharing the key k_c,
+sum_g T[h, g] (q_g . k_c(g)) = sum_c (sum_{g in c} T[h, g] q_g) . k_c, so the queries are mixed
+once a row (`lib.mix_heads`: a row of n_kv_heads * head_dim a head) and the generic kernel
+meets them with the keys of all kv heads laid end to end (`key_heads`).
 """
 from __future__ import annotations
 
@@ -77,8 +83,12 @@ class Attention:
             "k_proj.weight": ParamSpec((spec.kv_width, hidden)),
             "v_proj.weight": ParamSpec((spec.v_width, hidden)),
             "o_proj.weight": ParamSpec((hidden, spec.out_width)),
-            "o_proj.bias": ParamSpec((hidden,), optional=True),
         }
+        if spec.o_bias is not False:
+            params["o_proj.bias"] = ParamSpec((hidden,), optional=spec.o_bias is not True)
+        if spec.talking_heads:
+            params["talk"] = ParamSpec((spec.n_heads, spec.n_heads), init="near_identity",
+                                       scale=0.2)
         if spec.qkv_bias is not False:
             required = spec.qkv_bias is True
             params["q_proj.bias"] = ParamSpec((spec.q_width,), optional=not required)
@@ -106,9 +116,10 @@ class Attention:
         step."""
         group = spec.n_heads // max(1, spec.n_kv_heads)
         fast = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and MATRIX_CORE_ATTENTION
+                and not spec.talking_heads
                 and lib.attention_decode_mfma_supported(spec.head_dim, group))
         return ("rope_store", "attention_mfma" if fast else "attention_generic",
-                *Linear.kernel_libraries(dtype))
+                *(("head_ops",) if spec.talking_heads else ()), *Linear.kernel_libraries(dtype))
 
     @classmethod
     def check(cls, spec):
@@ -132,6 +143,14 @@ class Attention:
             if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
                 raise ValueError("attention: head_dim must be a multiple of 16 between 16 and "
                                  f"256, got {spec.head_dim}")
+        if spec.sink and spec.unit_sink:
+            raise ValueError("attention: a learned sink and a sink of 1 exclude each other")
+        if spec.talking_heads and spec.n_kv_heads * spec.head_dim > 1024:
+            raise ValueError("attention: with talking heads the keys of all kv heads of a "
+                             "position may hold 1024 elements at most, got "
+                             f"{spec.n_kv_heads * spec.head_dim}")
+        if spec.talking_heads and spec.distance_slope_range is not None:
+            raise ValueError("attention: talking heads with a distance term are not implemented")
         if spec.window is not None and spec.window < 1:
             raise ValueError("attention: a window must be at least 1")
         if spec.chunk is not None and spec.chunk < 1:
@@ -170,10 +189,15 @@ class Attention:
             self.slopes = torch.pow(2.0, exponent).to(device=device, dtype=torch.float32).contiguous()
         if spec.sink:
             self.sinks = params["sink"].to(device=device, dtype=torch.float32).contiguous()
+        elif spec.unit_sink:      # a sink of score 0: e^0 = 1 joins the denominator
+            self.sinks = torch.zeros(spec.n_heads, dtype=torch.float32, device=device)
+        self.talk = None
+        if spec.talking_heads:
+            self.talk = params["talk"].to(device=device, dtype=torch.float32).contiguous()
         # the matrix-core kernels take bfloat16 with head sizes 64 and 128 and values as wide
         # as the keys; every other case runs the generic kernel
         self.matrix_cores = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and
-                            MATRIX_CORE_ATTENTION and
+                            MATRIX_CORE_ATTENTION and self.talk is None and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
         # chunk, slopes, sink: what the kernels take beyond a window
         self.extras = dict(chunk=spec.chunk, slopes=self.slopes, sinks=self.sinks)
@@ -330,8 +354,15 @@ class Attention:
                 qkv, self.q_norm, self.k_norm, spec.qk_norm_eps, self.position.table,
                 meta.row_pos, meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads,
                 spec.n_kv_heads, spec.head_dim, write_cache=entry.writes_cache)
+        if self.talk is not None:
+            # the queries mixed over heads, one part for every kv head's keys
+            mixed = ctx.buffer("attn.q_mixed", (n, spec.q_width * spec.n_kv_heads))
+            lib.mix_heads(q, self.talk, mixed, spec.n_heads, spec.n_kv_heads, spec.head_dim)
+            ctx.release(q)
+            q = mixed
         out = ctx.buffer("attn.out", (n, spec.out_width))
-        more = dict(value_dim=spec.v_dim, **self.extras)
+        more = dict(value_dim=spec.v_dim, key_heads=1 if self.talk is None else spec.n_kv_heads,
+                    **self.extras)
         part_o = part_ml = None
         if ctx.decode:
             splits, waves, heads = self._decode_launch_for(ctx.n_seqs, ctx.context_bound)

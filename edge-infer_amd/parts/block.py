@@ -182,3 +182,115 @@ class OutputNormBlock:
         if self.narrow:
             ctx.notes[self.CAST_NOTE] = (x, index)
         return None
+
+
+class SandwichBlock:
+    """x += s * norm1b(mixer(norm1(x))); x += s * norm2b(feed_forward(norm2(x))): a norm before
+    and a norm after every sublayer, and a multiplier s (`residual_scale`) on what is added.  A
+    layer may have no feed-forward (then it has no second pair of norms either).
+
+    The multiplier is folded into the float32 weights of the norms on the outputs when the
+    block is built.  The norm on the mixer's output, the addition and the feed-forward's input
+    norm are one kernel; everything is added when the block returns, so it returns no pending
+    delta and follows only blocks that do the same."""
+
+    capture_safe = True      # nothing of its own besides its parts' kernels
+
+    def members(self):
+        return tuple(part for part in (self.norm1, self.mixer, self.norm1b, self.norm2, self.ffn,
+                                       self.norm2b) if part is not None)
+
+    @classmethod
+    def _owners(cls, layer_spec):
+        norm_cls = lookup("norm", layer_spec.norm.kind)
+        owners = [("norm1", norm_cls, layer_spec.norm),
+                  ("mixer", lookup("mixer", layer_spec.mixer.kind), layer_spec.mixer),
+                  ("norm1b", norm_cls, layer_spec.norm)]
+        if layer_spec.feed_forward is not None:
+            owners += [("norm2", norm_cls, layer_spec.norm),
+                       ("ffn", lookup("feed_forward", layer_spec.feed_forward.kind),
+                        layer_spec.feed_forward),
+                       ("norm2b", norm_cls, layer_spec.norm)]
+        return owners
+
+    @classmethod
+    def parameters(cls, layer_spec, hidden):
+        params = {}
+        for prefix, owner, spec in cls._owners(layer_spec):
+            for name, param in owner.parameters(spec, hidden).items():
+                params[f"{prefix}.{name}"] = param
+        if layer_spec.feed_forward is None:
+            # a checkpoint may still hold the second pair of norms of a layer without a
+            # feed-forward; they are taken and have no use
+            norm_cls = lookup("norm", layer_spec.norm.kind)
+            for prefix in ("norm2", "norm2b"):
+                for name, param in norm_cls.parameters(layer_spec.norm, hidden).items():
+                    params[f"{prefix}.{name}"] = ParamSpec(param.shape, init=param.init,
+                                                           optional=True)
+        return params
+
+    @classmethod
+    def mixer_spec(cls, layer_spec):
+        return layer_spec.mixer
+
+    @classmethod
+    def kernel_libraries(cls, layer_spec, dtype):
+        names = ["rowwise"]
+        for _, owner, spec in cls._owners(layer_spec):
+            ask = getattr(owner, "kernel_libraries", None)
+            if ask is not None:
+                names.extend(ask(spec, dtype))
+        return tuple(names)
+
+    def __init__(self, layer_spec, hidden, params, dtype, device, positions):
+        def sub(prefix):
+            return {name[len(prefix) + 1:]: tensor for name, tensor in params.items()
+                    if name.startswith(prefix + ".")}
+        norm_cls = lookup("norm", layer_spec.norm.kind)
+        if not hasattr(norm_cls, "norm_add"):
+            raise ValueError(f"norm kind '{layer_spec.norm.kind}' cannot sit on a sublayer's output")
+        scale = float(layer_spec.residual_scale)
+
+        def after(prefix):
+            """The norm on a sublayer's output, with the multiplier in its weight."""
+            norm = norm_cls(layer_spec.norm, hidden, sub(prefix), dtype, device)
+            if scale != 1.0:
+                norm.weight = (norm.weight * scale).contiguous()
+            return norm
+        self.norm1 = norm_cls(layer_spec.norm, hidden, sub("norm1"), dtype, device)
+        self.mixer = lookup("mixer", layer_spec.mixer.kind)(
+            layer_spec.mixer, hidden, sub("mixer"), dtype, device, positions=positions)
+        self.norm1b = after("norm1b")
+        self.norm2 = self.ffn = self.norm2b = None
+        if layer_spec.feed_forward is not None:
+            self.norm2 = norm_cls(layer_spec.norm, hidden, sub("norm2"), dtype, device)
+            self.ffn = lookup("feed_forward", layer_spec.feed_forward.kind)(
+                layer_spec.feed_forward, hidden, sub("ffn"), dtype, device)
+            self.norm2b = after("norm2b")
+        # the fused kernel takes two plain RMS norms of one eps
+        self.fused = all(hasattr(norm, "weight") and hasattr(norm, "eps")
+                         for norm in (self.norm1b, self.norm2) if norm is not None)
+
+    def forward(self, ctx, residual, pending, entry):
+        if pending is not None:
+            raise ValueError("sandwich: a delta of the block before is still pending; this "
+                             "arrangement follows only blocks that add everything themselves")
+        h = self.norm1.add_norm(ctx, residual, None, "block.h", write_residual=False)
+        a = self.mixer.forward(ctx, h, entry)
+        ctx.release(h)
+        if self.ffn is None:
+            self.norm1b.norm_add(ctx, residual, a)
+            ctx.release(a)
+            return None
+        if self.fused:
+            h2 = ctx.buffer("block.h", tuple(residual.shape))
+            lib.norm_add_norm(residual, a, self.norm1b.weight, self.norm2.weight, self.norm2.eps, h2)
+        else:
+            self.norm1b.norm_add(ctx, residual, a)
+            h2 = self.norm2.add_norm(ctx, residual, None, "block.h", write_residual=False)
+        ctx.release(a)
+        f = self.ffn.forward(ctx, h2)
+        ctx.release(h2)
+        self.norm2b.norm_add(ctx, residual, f)
+        ctx.release(f)
+        return None

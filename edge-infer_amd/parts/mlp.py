@@ -1,4 +1,5 @@
-"""Feed-forward parts.  `GatedMLP`: down(silu(gate(x)) * up(x)); `DenseMLP`:
+"""Feed-forward parts.  `GatedMLP`: down(act(gate(x)) * up(x)) with act silu or the tanh form
+of gelu; `DenseMLP`:
 down(act(up(x))) with act one of relu squared, relu, silu, tanh-gelu.
 
 The gated one:
@@ -46,8 +47,9 @@ class GatedMLP:
         }
 
     def __init__(self, spec, hidden, params, dtype, device):
-        if spec.activation != "silu":
-            raise ValueError(f"gated_mlp: activation '{spec.activation}' is not implemented")
+        if spec.activation not in lib.GATE_ACTIVATIONS:
+            raise ValueError(f"gated_mlp: activation '{spec.activation}' is not implemented; "
+                             f"known: {sorted(lib.GATE_ACTIVATIONS)}")
         self.spec = spec
         gate, up = params["gate_proj.weight"], params["up_proj.weight"]
         inter = spec.intermediate_size
@@ -74,11 +76,13 @@ class GatedMLP:
 
     def forward(self, ctx, x):
         n = x.shape[0]
-        act = self.gate_up.forward_gated(ctx, x, "mlp.act") if self.strip else None
+        # (the few-rows product that applies the gate itself knows silu only)
+        act = (self.gate_up.forward_gated(ctx, x, "mlp.act")
+               if self.strip and self.spec.activation == "silu" else None)
         if act is None:
             gate_up = self.gate_up.forward(ctx, x, "mlp.gate_up")
             act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
-            lib.swiglu(gate_up, act, self.strip)
+            lib.swiglu(gate_up, act, self.strip, self.spec.activation)
             ctx.release(gate_up)
         out = self.down.forward(ctx, act, "mlp.down")
         ctx.release(act)

@@ -39,3 +39,19 @@ class NoPosition:
         self.spec = spec
         self.table = None
         self.max_positions = None
+
+
+class RotaryFrequencies:
+    """Rotation of neighbouring pairs (2i, 2i + 1) by the angle position * theta^(-2i / dim):
+    the kernels multiply the float32 position by the float32 frequency and take cosine and
+    sine themselves, so there is no table and no position that is too far.  The frequencies
+    are float64 powers rounded once."""
+    def __init__(self, spec, device):
+        if spec.dim % 2 or spec.dim < 2:
+            raise ValueError("rotary dimension must be even and at least 2")
+        self.spec = spec
+        exponent = -2.0 * torch.arange(spec.dim // 2, dtype=torch.float64) / float(spec.dim)
+        frequencies = torch.pow(torch.tensor(float(spec.theta), dtype=torch.float64), exponent)
+        self.frequencies = frequencies.to(torch.float32).to(device).contiguous()
+        self.table = None
+        self.max_positions = None

@@ -23,7 +23,7 @@ import torch
 class ParamSpec:
     """One parameter a part expects.  `init` chooses the random-weights law:
     "normal" (N(0, scale), scale 0.02 unless given) for matrices and tables, "norm"
-    (1 + U(-0.1, 0.1)), "uniform" (U(low, high)).
+    (1 + U(-0.1, 0.1)), "uniform" (U(low, high)), "near_identity" (I + N(0, scale)).
     `optional`: taken when the checkpoint holds it, no error when it does not (the
     reference's optional projection biases, runtime/include/models/qwen3_model.hpp:371-403)."""
     shape: Tuple[int, ...]

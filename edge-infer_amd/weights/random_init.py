@@ -25,6 +25,9 @@ def random_tensor(spec: ParamSpec, generator: torch.Generator, device="cpu",
     elif spec.init == "uniform":
         value = spec.low + (spec.high - spec.low) * torch.rand(
             shape, generator=generator, device=device, dtype=torch.float32)
+    elif spec.init == "near_identity":      # square matrices that mix a little
+        value = torch.eye(shape[0], shape[1], device=device, dtype=torch.float32) + \
+            torch.randn(shape, generator=generator, device=device, dtype=torch.float32) * spec.scale
     else:
         raise ValueError(f"unknown initialisation '{spec.init}'")
     return value.to(dtype)
