@@ -95,7 +95,10 @@ class GatedMLPSpec:
     """down(act(gate(x)) * up(x))."""
     kind: str = "gated_mlp"
     intermediate_size: int = 0
-    activation: str = "silu"
+    activation: str = "silu"      # of the gate: "silu" or "gelu_tanh"
+    # biases of the three projections: None: taken when the checkpoint holds them, True: it
+    # must hold them, False: it must not
+    bias: Optional[bool] = None
 
 
 @dataclass(frozen=True)

@@ -287,7 +287,8 @@ class ZadenexConfig:
         layers = tuple(
             LayerSpec(block="sandwich", norm=norm, mixer=self._mixer_spec(layer.mixer),
                       feed_forward=None if layer.ff is None
-                      else GatedMLPSpec(intermediate_size=layer.ff, activation="gelu_tanh"),
+                      else GatedMLPSpec(intermediate_size=layer.ff, activation="gelu_tanh",
+                                        bias=True),
                       residual_scale=self.residual_mult)
             for layer in self.layers)
         loop = None if self.loop is None else LoopSpec(*self.loop)

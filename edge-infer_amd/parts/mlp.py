@@ -37,14 +37,18 @@ class GatedMLP:
 
     @classmethod
     def parameters(cls, spec, hidden):
-        return {
+        params = {
             "gate_proj.weight": ParamSpec((spec.intermediate_size, hidden)),
             "up_proj.weight": ParamSpec((spec.intermediate_size, hidden)),
             "down_proj.weight": ParamSpec((hidden, spec.intermediate_size)),
-            "gate_proj.bias": ParamSpec((spec.intermediate_size,), optional=True),
-            "up_proj.bias": ParamSpec((spec.intermediate_size,), optional=True),
-            "down_proj.bias": ParamSpec((hidden,), optional=True),
         }
+        wanted = getattr(spec, "bias", None)
+        if wanted is not False:
+            optional = wanted is not True
+            params["gate_proj.bias"] = ParamSpec((spec.intermediate_size,), optional=optional)
+            params["up_proj.bias"] = ParamSpec((spec.intermediate_size,), optional=optional)
+            params["down_proj.bias"] = ParamSpec((hidden,), optional=optional)
+        return params
 
     def __init__(self, spec, hidden, params, dtype, device):
         if spec.activation not in lib.GATE_ACTIVATIONS:

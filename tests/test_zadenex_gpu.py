@@ -1,0 +1,362 @@
+"""The Zadenex decoder in the engine against the plain implementation (`plain_zadenex`), in
+float32 and bfloat16: whole prompts, prompts then tokens one by one, portions down to two
+tokens, batches of unequal requests with slots and pages used again, long decoding over
+window edges and page borders, the first tokens of a sequence, a token far back, greedy
+generation through the entry point, and the framework's own random-weights folder."""
+import json
+
+import pytest
+import torch
+
+import plain_zadenex as plain
+from helpers import assert_close_bf16, assert_close_f32
+from zadenex_helpers import CONFIGS, ids, sharp_weights, tensor_shapes, write_folder
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+NAMES = ["A", "B", "C", "D"]
+LENGTHS = {"A": [150, 1, 49, 75], "B": [210, 2, 101, 64], "C": [200, 3, 130, 65],
+           "D": [140, 1, 5, 66]}
+# bfloat16 engine against the float64 oracle on these order-one weights: root-mean-square
+# error relative to the logits' root-mean-square, and largest error relative to the largest
+# logit (two norms a sublayer, a recurrent state and up to seven layer runs round more often
+# than the layers of the first architecture's tests)
+BF16_RMS, BF16_MAX = 4e-2, 12e-2
+
+
+def close(dtype, actual, expected, what):
+    if dtype == "float32":
+        return assert_close_f32(actual, expected, what)
+    return assert_close_bf16(actual, expected, what, rms_rel=BF16_RMS, max_rel=BF16_MAX)
+
+
+@pytest.fixture(scope="module")
+def weights():
+    return {name: sharp_weights(CONFIGS[name], seed=20 + i) for i, name in enumerate(NAMES)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory, weights):
+    root = tmp_path_factory.mktemp("zadenex")
+    return {name: write_folder(root / name, CONFIGS[name], weights[name]) for name in NAMES}
+
+
+@pytest.fixture(scope="module")
+def models(folders):
+    import edge_infer_amd as ei
+    cache = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in cache:
+            cache[(name, dtype)] = ei.load_model(folders[name], dtype=dtype)
+        return cache[(name, dtype)]
+    return get
+
+
+def requests_for(name, seed=5):
+    return [ids(CONFIGS[name]["vocab"], n, seed + i) for i, n in enumerate(LENGTHS[name])]
+
+
+@pytest.fixture(scope="module")
+def references(weights):
+    return {name: [plain.forward(CONFIGS[name], weights[name], r) for r in requests_for(name)]
+            for name in NAMES}
+
+
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_whole_prompts(models, references, name, dtype):
+    import edge_infer_amd as ei
+    session = ei.Session(models(name, dtype), max_tokens=512)
+    for request, ref in zip(requests_for(name), references[name]):
+        slot = session.begin()
+        logits = session.step([(slot, request, list(range(len(request))))])
+        close(dtype, logits, ref, f"{name} {dtype} whole {len(request)}")
+        session.end(slot)
+    session.cache.check()
+
+
+def test_the_stream_after_every_layer_run(models, weights):
+    """The float32 stream after each run of a layer (a looped layer counts each time) is the
+    oracle's."""
+    import edge_infer_amd as ei
+    model = models("A", "float32")
+    request = requests_for("A")[2]
+    _, kept = plain.forward(CONFIGS["A"], weights["A"], request, keep_layers=True)
+    seen = []
+    originals = [layer.forward for layer in model.layers]
+    try:
+        for layer, original in zip(model.layers, originals):
+            def watched(ctx, residual, pending, entry, original=original):
+                out = original(ctx, residual, pending, entry)
+                seen.append(residual.clone())
+                return out
+            layer.forward = watched
+        session = ei.Session(model, max_tokens=128, graphs=False)
+        session.step([(session.begin(), request, [])])
+    finally:
+        for layer in model.layers:
+            del layer.forward
+    assert len(seen) == kept.shape[0] == 1 + 3 * 2 + 1
+    for run, (got, want) in enumerate(zip(seen, kept)):
+        assert_close_f32(got, want, f"stream after run {run}")
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_prompt_then_tokens_one_by_one(models, references, name, dtype, graphs):
+    """The decoded tokens pass window edges and a page border (64, 128)."""
+    import edge_infer_amd as ei
+    session = ei.Session(models(name, dtype), max_tokens=512, graphs=graphs)
+    for request, ref in zip(requests_for(name), references[name]):
+        cut = max(1, len(request) - 60)
+        slot = session.begin()
+        rows = [session.step([(slot, request[:cut], [cut - 1])])]
+        rows += [session.step([(slot, [token], [0])]) for token in request[cut:]]
+        close(dtype, torch.cat(rows), ref[cut - 1:], f"{name} {dtype} tail of {len(request)}")
+        session.end(slot)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("sizes", [(2, 2, 3, 2), (1, 5, 64, 2, 7), (63, 2, 65), (20, 100, 3)])
+def test_portions(models, references, name, dtype, sizes):
+    """A prompt cut into portions (the given sizes in turn, down to two tokens and one): every
+    position's logits are those of the whole prompt."""
+    import edge_infer_amd as ei
+    session = ei.Session(models(name, dtype), max_tokens=512)
+    request, ref = requests_for(name)[0], references[name][0]
+    slot = session.begin()
+    rows, at, turn = [], 0, 0
+    while at < len(request):
+        take = min(sizes[turn % len(sizes)], len(request) - at)
+        rows.append(session.step([(slot, request[at:at + take], list(range(take)))]))
+        at, turn = at + take, turn + 1
+    close(dtype, torch.cat(rows), ref, f"{name} {dtype} portions {sizes}")
+    session.end(slot)
+
+
+def test_float32_logits_do_not_depend_on_the_cut(models):
+    """Whole, in portions and token by token: the same float32 logits to the last bits."""
+    import edge_infer_amd as ei
+    model = models("A", "float32")
+    request = requests_for("A")[0][:100]
+    session = ei.Session(model, max_tokens=512)
+
+    def run(sizes):
+        slot = session.begin()
+        rows, at = [], 0
+        for take in sizes:
+            rows.append(session.step([(slot, request[at:at + take], list(range(take)))]))
+            at += take
+        session.end(slot)
+        return torch.cat(rows)
+    whole = run([100])
+    for sizes in ([37, 63], [2] * 50, [99, 1], [1] * 100):
+        got = run(sizes)
+        assert (got - whole).abs().max().item() <= 2e-6 * whole.abs().max().item(), sizes
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_batches_of_unequal_requests_with_slots_and_pages_used_again(models, references, name, dtype):
+    """Requests of unequal lengths start together and are decoded together; the shorter end
+    earlier and their slots and pages go back; a second and a third batch then run in what was
+    freed (the cache has room for little more than one batch)."""
+    import edge_infer_amd as ei
+    requests, refs = requests_for(name), references[name]
+    tail = 20
+    session = ei.Session(models(name, dtype), max_tokens=64 * 12, max_seqs=4)
+    for batch in ([0, 1, 2, 3], [3, 2, 0], [1, 0, 3, 2]):
+        slots = {i: session.begin() for i in batch}
+        cuts = {i: max(1, len(requests[i]) - tail) for i in batch}
+        got = {i: [] for i in batch}
+        logits = session.step([(slots[i], requests[i][:cuts[i]], [cuts[i] - 1]) for i in batch])
+        for row, i in enumerate(batch):
+            got[i].append(logits[row:row + 1])
+        at = dict(cuts)
+        live = [i for i in batch if at[i] < len(requests[i])]
+        for i in batch:
+            if i not in live:
+                session.end(slots[i])
+        while live:
+            logits = session.step([(slots[i], [requests[i][at[i]]], [0]) for i in live])
+            for row, i in enumerate(live):
+                got[i].append(logits[row:row + 1])
+                at[i] += 1
+            for i in [i for i in live if at[i] == len(requests[i])]:
+                session.end(slots[i])
+                live.remove(i)
+        for i in batch:
+            close(dtype, torch.cat(got[i]), refs[i][cuts[i] - 1:],
+                  f"{name} {dtype} request {i} in batch {batch}")
+        session.cache.check()
+    assert session.cache.slots.n_free == 4
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_long_decoding_from_the_first_token(models, weights, name, dtype):
+    """One token, then 299 more one by one, from graphs: every window's edge and four page
+    borders are passed while decoding, and the state is carried 300 times."""
+    import edge_infer_amd as ei
+    request = ids(CONFIGS[name]["vocab"], 300, 77)
+    ref = plain.forward(CONFIGS[name], weights[name], request)
+    session = ei.Session(models(name, dtype), max_tokens=320)
+    slot = session.begin()
+    rows = [session.step([(slot, [token], [0])]) for token in request]
+    close(dtype, torch.cat(rows), ref, f"{name} {dtype} 300 tokens one by one")
+    assert session.graphs and session.graph_replays > 250
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_a_failed_step_leaves_the_state_as_it_was(models, references, graphs):
+    """The matrix memory's state has two versions a slot: a step that fails after its layers
+    have run (here the head raises, once in a prompt portion and once in a decode step) has
+    written the other version only, so the same step again gives what a run without the
+    failure gives."""
+    import edge_infer_amd as ei
+    model = models("A", "float32")
+    request, ref = requests_for("A")[0], references["A"][0]
+    session = ei.Session(model, max_tokens=512, graphs=graphs)
+    assert session.cache.two_versions and all(c is None for c in session.cache._state_copies)
+    slot = session.begin()
+    rows = [session.step([(slot, request[:40], list(range(40)))])]
+    whole = type(model).logits
+    failures = []
+
+    def failing(self, ctx, hidden):
+        if not failures:
+            failures.append(ctx.n_rows)
+            raise RuntimeError("forced failure after the layers have run")
+        return whole(self, ctx, hidden)
+    try:
+        type(model).logits = failing
+        with pytest.raises(RuntimeError, match="forced failure"):
+            session.step([(slot, request[40:90], list(range(50)))])
+        assert session.length(slot) == 40
+        rows.append(session.step([(slot, request[40:90], list(range(50)))]))
+        failures.clear()       # (the first decode step: the one that runs eagerly before a graph is made)
+        with pytest.raises(RuntimeError, match="forced failure"):
+            session.step([(slot, request[90:91], [0])])
+        for t in range(90, 100):
+            rows.append(session.step([(slot, request[t:t + 1], [0])]))
+    finally:
+        type(model).logits = whole
+    close("float32", torch.cat(rows), ref[:100], "after failed steps")
+
+
+@pytest.mark.parametrize("name", ["A", "B", "D"])
+def test_a_token_far_back_shows(tmp_path, name):
+    """Two prompts that differ in their third token alone still differ at position 400, by far
+    more than the tolerance (through the matrix memories, which here forget slowly, and
+    through latent attention, which sees every earlier position), and the engine follows the
+    oracle for both, whole, in portions and decoded."""
+    import edge_infer_amd as ei
+    cfg = CONFIGS[name]
+    tensors = sharp_weights(cfg, seed=31, long_memory=True)
+    model = ei.load_model(write_folder(tmp_path / "slow", cfg, tensors), dtype="float32")
+    base = ids(cfg["vocab"], 401, 3)
+    other = list(base)
+    other[2] = (base[2] + 1) % cfg["vocab"]
+    refs = [plain.forward(cfg, tensors, r)[-1:] for r in (base, other)]
+    gap = (refs[0] - refs[1]).abs().max().item() / refs[0].abs().max().item()
+    assert gap > 1e-3, f"the test's weights do not carry the third token to the end ({gap:.1e})"
+    session = ei.Session(model, max_tokens=1024)
+    for request, ref in zip((base, other), refs):
+        slot = session.begin()
+        close("float32", session.step([(slot, request, [400])]), ref, "far token, whole")
+        session.end(slot)
+        slot = session.begin()
+        session.step([(slot, request[:130], [])])
+        session.step([(slot, request[130:390], [])])
+        for token in request[390:400]:
+            session.step([(slot, [token], [])])
+        close("float32", session.step([(slot, request[400:], [0])]), ref, "far token, decoded")
+        session.end(slot)
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_greedy_generation_through_the_entry_point(models, weights, name):
+    """`Session.generate_batch` (the scheduler, sampler and step function together) gives the
+    oracle's greedy tokens in float32."""
+    import edge_infer_amd as ei
+    cfg = CONFIGS[name]
+    prompts = [ids(cfg["vocab"], n, 40 + n) for n in (5, 1, 30)]
+    session = ei.Session(models(name, "float32"), max_tokens=512, max_seqs=3)
+    got = session.generate_batch(prompts, max_new_tokens=12, temperature=0.0)
+    for prompt, tokens in zip(prompts, got):
+        sequence = list(prompt)
+        for token in tokens:
+            logits = plain.forward(cfg, weights[name], sequence)[-1]
+            best = logits.argmax().item()
+            if token != best:       # only a tie within float32's reach may differ
+                assert (logits[best] - logits[token]).item() <= 2e-5 * logits.abs().max().item()
+            sequence.append(token)
+        assert len(tokens) == 12
+
+
+def test_model_type_through_the_python_entry(folders, weights):
+    from edge_infer_amd.api import Model
+    model = Model.from_pretrained(folders["A"], "zadenex_fp32")
+    session = model.new_session(capacity=128, max_batch=2)
+    prompt = ids(CONFIGS["A"]["vocab"], 9, 1)
+    tokens = session.generate(prompt, None, max_length=len(prompt) + 4, temperature=0.0)
+    logits = plain.forward(CONFIGS["A"], weights["A"], prompt)[-1]
+    assert tokens[0] == logits.argmax().item() and len(tokens) == 4
+    with pytest.raises(ValueError, match="names the family"):
+        Model.from_pretrained(folders["A"], "qwen3_bf16")
+
+
+def test_random_weights_folder_of_the_framework(tmp_path):
+    """`write_model_folder` writes a Zadenex folder that reads back to the same configuration
+    and runs; its tensors carry the checkpoint's names."""
+    import edge_infer_amd as ei
+    from safetensors.torch import load_file
+    cfg = ei.config.ZadenexConfig.from_dict(CONFIGS["B"])
+    folder = ei.write_model_folder(tmp_path / "random", cfg, seed=2)
+    assert ei.read_config(folder)[1] == cfg
+    tensors = load_file(str(folder / "model.safetensors"))
+    shapes = {k: shape for k, (shape, _) in tensor_shapes(CONFIGS["B"]).items()}
+    assert set(tensors) <= set(shapes)       # (the unused norms of a layer without a feed-forward are left out)
+    assert all(tuple(v.shape) == tuple(shapes[k]) for k, v in tensors.items())
+    model = ei.load_model(folder, dtype="bfloat16")
+    session = ei.Session(model, max_tokens=128)
+    slot = session.begin()
+    request = ids(CONFIGS["B"]["vocab"], 70, 9)
+    logits = session.step([(slot, request, [69])])
+    ref = plain.forward(json.loads((folder / "config.json").read_text()), tensors, request)[-1:]
+    close("bfloat16", logits, ref, "random folder")
+
+
+def test_the_replay_program_runs_a_zadenex_folder(folders, weights, tmp_path):
+    """`bin/trace_run` chooses the model class by config.json and writes the step's logits."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    import numpy as np
+    root = Path(__file__).resolve().parents[1]
+    vocab = CONFIGS["A"]["vocab"]
+    one, two = ids(vocab, 30, 8), ids(vocab, 12, 9)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": one[:28], "want": [0, 27]},
+                                     {"id": "y", "tokens": two[:11], "want": [10]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": one[28:29], "want": []},
+                                     {"id": "y", "tokens": two[11:], "want": [0]}], "end": ["y"]},
+             {"step": 2, "entries": [{"id": "x", "tokens": one[29:], "want": [0]}], "end": ["x"]}]
+    done = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model",
+                           str(folders["A"]), "--dtype", "float32", "--out", str(tmp_path),
+                           "--max-tokens", "64"], input="\n".join(json.dumps(s) for s in steps),
+                          capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert [l for l in done.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    ref_one = plain.forward(CONFIGS["A"], weights["A"], one)
+    ref_two = plain.forward(CONFIGS["A"], weights["A"], two)
+    first = torch.from_numpy(np.fromfile(tmp_path / "0.f32", dtype="<f4").reshape(3, vocab))
+    second = torch.from_numpy(np.fromfile(tmp_path / "1.f32", dtype="<f4").reshape(1, vocab))
+    last = torch.from_numpy(np.fromfile(tmp_path / "2.f32", dtype="<f4").reshape(1, vocab))
+    assert_close_f32(first, torch.cat([ref_one[[0, 27]], ref_two[[10]]]), "replayed prompts")
+    assert_close_f32(second, ref_two[11:], "replayed token of the short request")
+    assert_close_f32(last, ref_one[29:], "replayed token")
