@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
                     [--shape 8b|0.6b|32b] [--only decode|prefill|generate] [--prompt P]
-                    [--with-32b] [--peaks] [--design tirurax [--design-shape 1k|2k|4k]]
+                    [--with-32b] [--peaks] [--design tirurax|zadenex [--design-shape 1k|2k|4k]]
 
 Prints one JSON line.  `value` is decoded tokens per second at the given batch after
 512-token prompts (one step = one decode step of the whole batch: the model, greedy
@@ -24,7 +24,10 @@ of a decode step, and what a graph of as many launches of a kernel that does not
 (one prompt of 2,048 tokens, and 8 of 512) and decode (batch 1, 8 and 64 after 512-token
 prompts) of a Tirurax model of real layer sizes (gated-delta and chunked-attention layers in
 turn, dense feed-forward of four widths) beside a Qwen3 model of the same width, layers,
-heads and parameter count, as one JSON line.
+heads and parameter count, as one JSON line.  `--design zadenex` does the same for a Zadenex
+model (matrix-memory, latent-attention and window-attention layers whose scores are mixed over
+heads, gated feed-forward, one pass of a loop over the last six layers) beside the Tirurax
+model of the same width, layers, heads and parameter count.
 Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
 ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s; `measured_peaks` (and `--peaks` alone) say what
 a plain read kernel and a loop of matrix-core products reach on the GPU at hand, and the
@@ -363,6 +366,46 @@ def design_configs(shape):
     return new, old
 
 
+def zadenex_configs(shape):
+    """(Zadenex configuration, Tirurax configuration) of equal width, layers, heads, head size
+    and feed-forward parameters: a matrix-memory layer stands where a gated-delta layer stands,
+    latent and window attention in turn where chunked attention stands; the latent is four
+    head sizes wide, the rotated part half a head size."""
+    from edge_infer_amd.config import TiruraxConfig, ZadenexConfig
+    layers, width, d_heads, d_kv, a_heads, a_kv, dim, chunk, vocab = DESIGN_SHAPES[shape]
+    ff = 4 * width
+    gated = {"kind": "dense", "ff": (2 * ff // 3 + 255) // 256 * 256}
+    memory = {"type": "mlstm", "mixer": {"heads": d_heads, "dim": dim, "vdim": dim,
+                                         "gate_cap": 15.0}, "mlp": gated}
+    latent = {"type": "latent_attention",
+              "mixer": {"heads": a_heads, "dim": dim, "rot_dim": dim // 2, "vdim": dim,
+                        "kv_rank": 4 * dim, "q_rank": width // 2 + dim,
+                        "scale": (1.5 * dim) ** -0.5, "rot": {"base": 10000.0, "dims": dim // 2}},
+              "mlp": gated}
+    window = {"type": "attention", "mixer": {"heads": a_heads, "kv_heads": a_kv, "dim": dim,
+                                             "vdim": dim, "scale": dim ** -0.5,
+                                             "mask": {"size": chunk}},
+              "mlp": gated}
+    order = [memory if i % 2 == 0 else (latent if i % 4 == 1 else window) for i in range(layers)]
+    new = ZadenexConfig.from_dict({"architecture": "Zadenex", "vocab": vocab, "width": width,
+                                   "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+                                   "residual_mult": 0.5,
+                                   "loop": {"start": 2, "stop": layers, "times": 1},
+                                   "layers": order})
+    delta = {"type": "delta", "mixer": {"heads": d_heads, "kv_heads": d_kv, "dim": dim,
+                                        "vdim": dim, "conv": 4},
+             "mlp": {"kind": "dense", "ff": ff}}
+    attention = {"type": "attention", "mixer": {"heads": a_heads, "kv_heads": a_kv, "dim": dim,
+                                                "vdim": dim, "scale": dim ** -0.5,
+                                                "mask": {"size": chunk}},
+                 "mlp": {"kind": "dense", "ff": ff}}
+    old = TiruraxConfig.from_dict({"architecture": "Tirurax", "vocab": vocab, "width": width,
+                                   "norm": {"eps": 1e-6},
+                                   "layers": [delta if i % 2 == 0 else attention
+                                              for i in range(layers)]})
+    return new, old
+
+
 def measure_prompts(model, vocab, batch, tokens, repeats=3):
     """Best ms of one step over `batch` prompts of `tokens` tokens that start together."""
     import types
@@ -387,17 +430,25 @@ def measure_prompts(model, vocab, batch, tokens, repeats=3):
 
 
 def design_comparison(args):
-    """Prefill and decode of the Tirurax shape and of the Qwen3 model of equal size."""
+    """Prefill and decode of the design's shape and of the closest other model of equal size
+    (Tirurax beside Qwen3, Zadenex beside Tirurax)."""
     import types
     import torch
     import edge_infer_amd as ei
-    new, old = design_configs(args.design_shape)
+    if args.design == "zadenex":
+        new, old = zadenex_configs(args.design_shape)
+        which = {"zadenex": new, "tirurax": old}
+    else:
+        new, old = design_configs(args.design_shape)
+        which = {"tirurax": new, "qwen3": old}
     vocab = new.vocab
     sizes = types.SimpleNamespace(vocab_size=vocab)
-    record = {"only": "design", "design": "tirurax", "shape": args.design_shape,
+    record = {"only": "design", "design": args.design, "shape": args.design_shape,
               "dtype": args.dtype, "layers": len(new.layers), "width": new.width}
-    which = {"tirurax": new, "qwen3": old}
     if args.design_only:
+        if args.design_only not in which:
+            print(f"bench.py: --design {args.design} compares {' and '.join(which)}")
+            return 2
         which = {args.design_only: which[args.design_only]}
     for name, cfg in which.items():
         model = ei.random_model(cfg, seed=2, dtype=args.dtype)
@@ -446,11 +497,12 @@ def main():
                         help="leave the 32B shape (decode at batch 1 and 16, prefill) out of `points`")
     parser.add_argument("--peaks", action="store_true",
                         help="measure the read and matrix-core yardsticks only")
-    parser.add_argument("--design", choices=["tirurax"], default=None,
-                        help="measure this design beside the Qwen3 model of equal size instead "
-                             "of the default workload")
+    parser.add_argument("--design", choices=["tirurax", "zadenex"], default=None,
+                        help="measure this design beside the closest other model of equal size "
+                             "(tirurax beside qwen3, zadenex beside tirurax) instead of the "
+                             "default workload")
     parser.add_argument("--design-shape", choices=sorted(DESIGN_SHAPES), default="2k")
-    parser.add_argument("--design-only", choices=["tirurax", "qwen3"], default=None,
+    parser.add_argument("--design-only", choices=["zadenex", "tirurax", "qwen3"], default=None,
                         help="with --design: one of the two models only (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1:

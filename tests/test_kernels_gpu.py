@@ -588,12 +588,14 @@ def test_attention_prefill_on_the_matrix_cores_window_and_far_key(lib, window, k
         close(out, expected, torch.bfloat16)
 
 
-def test_attention_takes_any_head_size_up_to_256_and_refuses_more(lib):
+def test_attention_takes_any_head_size_up_to_512_and_refuses_more(lib):
     from edge_infer_amd.csrc.lib import KernelError
     out, expected = run_attention(lib, torch.float32, 2, 1, 24, [0], [70])
     close(out, expected, torch.float32)
-    with pytest.raises(KernelError, match="between 1 and 256"):
-        run_attention(lib, torch.float32, 2, 1, 512, [0], [4])
+    out, expected = run_attention(lib, torch.float32, 3, 1, 512, [0], [70])     # (beyond 64 KB of LDS)
+    close(out, expected, torch.float32)
+    with pytest.raises(KernelError, match="values of at most 512"):
+        run_attention(lib, torch.float32, 2, 1, 528, [0], [4])
 
 
 # ---------------------------------------------------------------------------
