@@ -75,6 +75,14 @@ _SIGNATURES = {
                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
                          c_int, c_int, c_int, c_void_p, c_void_p],
     },
+    "attention_wide": {
+        "ei_attn_wide_supported": [c_int, c_int, c_int],
+        "ei_attn_wide_positions": [c_int],
+        "ei_attention_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                              c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                              c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_int,
+                              c_int, c_int, c_void_p, c_void_p],
+    },
     "head_ops": {
         "ei_latent_down_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_float,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
@@ -541,6 +549,75 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
         key_heads, int(bool(values_in_keys)),
         None if gate is None else _gpu(gate, "gate", torch.float32), _stream())
     _check(lib, status, "attention")
+
+
+def attention_wide_supported(dtype, query_width: int, head_dim: int, value_dim: int) -> bool:
+    """Whether the matrix-core kernel for wide keys takes these sizes (asked without loading
+    its library): bfloat16, query rows (key_heads * head_dim) a multiple of 32 up to 1024, the
+    stored key head size a multiple of 8, values a multiple of 16 up to 512."""
+    return (dtype == torch.bfloat16 and 32 <= query_width <= 1024 and query_width % 32 == 0
+            and head_dim % 8 == 0 and 16 <= value_dim <= 512 and value_dim % 16 == 0)
+
+
+def attention_wide_positions(group: int) -> int:
+    """Positions of one sequence that a work item of `attention_wide` may hold: a block has
+    64 query rows, positions x heads of a kv group."""
+    return 64 // min(group, 64)
+
+
+def attention_wide(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos, row_seq,
+                   page_table, out, n_heads, n_kv_heads, head_dim, window=None, scale=None,
+                   n_splits=1, part_o=None, part_ml=None, value_dim=None, sinks=None, key_heads=1,
+                   values_in_keys=False, gate=None) -> None:
+    """bfloat16 attention on the matrix cores for wide keys (see attention_wide.hip); arguments
+    as `attention`'s."""
+    lib = library("attention_wide")
+    n = q.shape[0]
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    key_heads = int(key_heads)
+    if key_heads not in (1, n_kv_heads):
+        raise KernelError("attention_wide: key_heads must be 1 or the number of kv heads")
+    if not attention_wide_supported(q.dtype, key_heads * head_dim, head_dim, value_dim):
+        raise KernelError("attention_wide: these head sizes or this type are not supported")
+    if tuple(q.shape) != (n, n_heads * key_heads * head_dim) or \
+            tuple(out.shape) != (n, n_heads * value_dim):
+        raise KernelError("attention_wide: q must be [rows, heads * key_heads * head_dim] and out "
+                          "[rows, heads * value_dim]")
+    if tuple(k_pages.shape[1:]) != (n_kv_heads, PAGE_TOKENS, head_dim):
+        raise KernelError("attention_wide: key pages have the wrong shape")
+    if values_in_keys:
+        if value_dim > head_dim:
+            raise KernelError("attention_wide: values inside the keys cannot be wider than them")
+        v_pages = k_pages
+    elif tuple(v_pages.shape) != (k_pages.shape[0], n_kv_heads, PAGE_TOKENS, value_dim):
+        raise KernelError("attention_wide: value pages have the wrong shape")
+    if not (k_pages.dtype == v_pages.dtype == out.dtype == torch.bfloat16):
+        raise KernelError("attention_wide: q, cache and out must be bfloat16")
+    if item_seq.numel() < n_items or item_row0.numel() < n_items or item_npos.numel() < n_items:
+        raise KernelError("attention_wide: work item arrays shorter than n_items")
+    if sinks is not None and sinks.numel() != n_heads:
+        raise KernelError("attention_wide: sinks must have one value per query head")
+    if gate is not None and (gate.dtype != torch.float32 or gate.numel() != n * n_heads):
+        raise KernelError("attention_wide: the gate must be float32 [rows, heads]")
+    if n_splits > 1:
+        if part_o is None or part_ml is None or part_o.numel() < n * n_heads * n_splits * value_dim \
+                or part_ml.numel() < n * n_heads * n_splits * 2:
+            raise KernelError("attention_wide: split scratch missing or too small")
+    if scale is None:
+        scale = head_dim ** -0.5
+    status = lib.ei_attention_wide(
+        _gpu(q, "q"), _gpu(k_pages, "k_pages"), _gpu(v_pages, "v_pages"),
+        _gpu(item_seq, "item_seq", torch.int32), _gpu(item_row0, "item_row0", torch.int32),
+        _gpu(item_npos, "item_npos", torch.int32), n_items, _gpu(row_pos, "row_pos", torch.int32),
+        _gpu(row_seq, "row_seq", torch.int32), _gpu(page_table, "page_table", torch.int32),
+        page_table.shape[-1], _gpu(out, "out"),
+        None if part_o is None else _gpu(part_o, "part_o", torch.float32),
+        None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
+        n_kv_heads, head_dim, value_dim, int(window or 0),
+        None if sinks is None else _gpu(sinks, "sinks", torch.float32), float(scale), n_splits,
+        key_heads, int(bool(values_in_keys)),
+        None if gate is None else _gpu(gate, "gate", torch.float32), _stream())
+    _check(lib, status, "attention_wide")
 
 
 # ---------------------------------------------------------------------------

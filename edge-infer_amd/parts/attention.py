@@ -118,8 +118,19 @@ class Attention:
         fast = (dtype == torch.bfloat16 and spec.v_dim == spec.head_dim and MATRIX_CORE_ATTENTION
                 and not spec.talking_heads
                 and lib.attention_decode_mfma_supported(spec.head_dim, group))
-        return ("rope_store", "attention_mfma" if fast else "attention_generic",
-                *(("head_ops",) if spec.talking_heads else ()), *Linear.kernel_libraries(dtype))
+        kernels = "attention_mfma" if fast else "attention_generic"
+        if cls.wide_keys(spec, dtype):
+            kernels = "attention_wide"
+        return ("rope_store", kernels, *(("head_ops",) if spec.talking_heads else ()),
+                *Linear.kernel_libraries(dtype))
+
+    @classmethod
+    def wide_keys(cls, spec, dtype) -> bool:
+        """Whether this part runs the matrix-core kernel for wide keys: scores mixed over heads
+        (queries as wide as the keys of all kv heads together), bfloat16, sizes it takes."""
+        return (spec.talking_heads and MATRIX_CORE_ATTENTION and spec.chunk is None
+                and lib.attention_wide_supported(dtype, spec.n_kv_heads * spec.head_dim,
+                                                 spec.head_dim, spec.v_dim))
 
     @classmethod
     def check(cls, spec):
@@ -200,6 +211,7 @@ class Attention:
                             MATRIX_CORE_ATTENTION and self.talk is None and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
         # chunk, slopes, sink: what the kernels take beyond a window
+        self.wide = self.wide_keys(spec, dtype)
         self.extras = dict(chunk=spec.chunk, slopes=self.slopes, sinks=self.sinks)
         self.has_extras = spec.chunk is not None or self.slopes is not None or self.sinks is not None
         self.compute_units = lib.compute_units(device)     # the chip's size, for launch plans
@@ -207,6 +219,8 @@ class Attention:
 
     # the number of positions of one sequence that a prefill work item covers
     def positions_per_item(self, key_ways: int = 1):
+        if self.wide:
+            return lib.attention_wide_positions(self.group) if key_ways == 1 else 0
         if self.matrix_cores:          # the matrix-core prefill kernel takes the same cases
             return lib.attention_prefill_mfma_positions(self.group, key_ways)
         return lib.attention_positions_per_item(self.group) if key_ways == 1 else 0
@@ -231,7 +245,7 @@ class Attention:
     @property
     def plan_key(self):
         """Attention parts with equal keys plan the same sections."""
-        return ("attention", self.positions_per_item(), self.group, self.spec.n_kv_heads)
+        return ("attention", self.positions_per_item(), self.group, self.spec.n_kv_heads, self.wide)
 
     def _items_section(self, key_ways: int = 1):
         return f"attention.items{self.positions_per_item(key_ways)}"
@@ -380,11 +394,19 @@ class Attention:
                                           **self.extras)
             else:
                 item_seq, item_row0, item_npos, n_items = self._items(ctx, "attention.decode_items")
-                lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
-                              meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
-                              spec.n_kv_heads, spec.head_dim, window=spec.window,
-                              scale=self.scale, n_splits=splits, part_o=part_o, part_ml=part_ml,
-                              **more)
+                if self.wide:
+                    lib.attention_wide(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
+                                       meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
+                                       spec.n_kv_heads, spec.head_dim, window=spec.window,
+                                       scale=self.scale, n_splits=splits, part_o=part_o,
+                                       part_ml=part_ml, value_dim=spec.v_dim, sinks=self.sinks,
+                                       key_heads=spec.n_kv_heads)
+                else:
+                    lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
+                                  meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
+                                  spec.n_kv_heads, spec.head_dim, window=spec.window,
+                                  scale=self.scale, n_splits=splits, part_o=part_o,
+                                  part_ml=part_ml, **more)
         else:
             key_ways = self.prefill_key_ways([seq.count for seq in ctx.sequences])
             section = self._items_section(key_ways)
@@ -401,6 +423,12 @@ class Attention:
                                            scale=self.scale, key_ways=key_ways,
                                            pair_items=len({(seq.start, seq.count) for seq in ctx.sequences}) == 1,
                                            largest_item=largest, **self.extras)
+            elif self.wide:
+                lib.attention_wide(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
+                                   meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
+                                   spec.n_kv_heads, spec.head_dim, window=spec.window,
+                                   scale=self.scale, value_dim=spec.v_dim, sinks=self.sinks,
+                                   key_heads=spec.n_kv_heads)
             else:
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,

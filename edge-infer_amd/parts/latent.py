@@ -17,7 +17,9 @@ so the up-projections never touch the cache: a head's query is carried into the 
 whose key is the cached row [c | t] and whose value is that row's first kv_rank elements, and
 the value up-projection is applied to the head's weighted sum of latents.  The softmax's
 denominator may hold a learned sink per head.  Projections of x are one fused matrix
-[dq | dkv | g].  Kernels: `csrc/head_ops.hip`, `csrc/attention_generic.hip`.
+[dq | dkv | g].  Kernels: `csrc/head_ops.hip`; attention in bfloat16 on the matrix cores
+(`csrc/attention_wide.hip`: cache rows a multiple of 32 wide, latents a multiple of 16),
+otherwise, and in float32, `csrc/attention_generic.hip`.
 """
 from __future__ import annotations
 
@@ -27,7 +29,7 @@ import torch
 from ..csrc import lib
 from ..csrc.lib import PAGE_TOKENS
 from ..weights.loader import ParamSpec
-from .attention import MAX_SLICES, _decode_items
+from .attention import MATRIX_CORE_ATTENTION, MAX_SLICES, _decode_items
 from .base import KVRequest
 from .linear import Linear
 
@@ -66,8 +68,14 @@ class LatentAttention:
         return KVRequest(n_kv_heads=1, head_dim=spec.cache_width, value_dim=0)
 
     @classmethod
+    def on_matrix_cores(cls, spec, dtype) -> bool:
+        return MATRIX_CORE_ATTENTION and lib.attention_wide_supported(
+            dtype, spec.cache_width, spec.cache_width, spec.kv_rank)
+
+    @classmethod
     def kernel_libraries(cls, spec, dtype):
-        return ("head_ops", "attention_generic", *Linear.kernel_libraries(dtype))
+        attention = "attention_wide" if cls.on_matrix_cores(spec, dtype) else "attention_generic"
+        return ("head_ops", attention, *Linear.kernel_libraries(dtype))
 
     @classmethod
     def check(cls, spec):
@@ -107,11 +115,13 @@ class LatentAttention:
         self.frequencies = positions(spec.position).frequencies if r else None
         self.scale = spec.scale if spec.scale is not None else float(d + r) ** -0.5
         self.compute_units = lib.compute_units(device)
-        self.positions_per_item = lib.attention_positions_per_item(H)
+        self.wide = self.on_matrix_cores(spec, dtype)
+        self.positions_per_item = (lib.attention_wide_positions(H) if self.wide
+                                   else lib.attention_positions_per_item(H))
 
     @property
     def plan_key(self):
-        return ("latent_attention", self.positions_per_item)
+        return ("latent_attention", self.positions_per_item, self.wide)
 
     def plan_step(self, plan):
         """Work items of the attention kernel, [3, items]: sequence, first row, positions."""
@@ -131,8 +141,12 @@ class LatentAttention:
         """Slices of the key range in a decode step: enough blocks for about two a compute
         unit, never more than there are pages."""
         pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
-        blocks = n_seqs * ((self.spec.n_heads + 15) // 16)
-        wanted = (2 * self.compute_units + blocks - 1) // blocks
+        if self.wide:         # blocks of up to 64 heads, about one a compute unit
+            blocks = n_seqs * ((self.spec.n_heads + 63) // 64)
+            wanted = max(1, self.compute_units // blocks)
+        else:
+            blocks = n_seqs * ((self.spec.n_heads + 15) // 16)
+            wanted = (2 * self.compute_units + blocks - 1) // blocks
         return max(1, min(wanted, pages, MAX_SLICES))
 
     def forward(self, ctx, x, entry):
@@ -174,9 +188,10 @@ class LatentAttention:
         else:
             section = meta.section(f"latent.items{self.positions_per_item}")
         count = section.numel() // 3
-        lib.attention(q_wide, k_pages, None, section[:count], section[count:2 * count],
-                      section[2 * count:], count, meta.row_pos, meta.row_seq, page_table, mixed,
-                      H, 1, spec.cache_width, **common)
+        kernel = lib.attention_wide if self.wide else lib.attention
+        kernel(q_wide, k_pages, None, section[:count], section[count:2 * count],
+               section[2 * count:], count, meta.row_pos, meta.row_seq, page_table, mixed,
+               H, 1, spec.cache_width, **common)
         ctx.release(q_wide, gate, part_o, part_ml)
         out = ctx.buffer("latent.out", (n, spec.out_width))
         lib.head_matmul(mixed, self.v_up, out, H, x_head=rank, x_first=0,

@@ -15,9 +15,9 @@ from zadenex_helpers import CONFIGS, ids, sharp_weights, tensor_shapes, write_fo
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-NAMES = ["A", "B", "C", "D"]
+NAMES = ["A", "B", "C", "D", "E"]
 LENGTHS = {"A": [150, 1, 49, 75], "B": [210, 2, 101, 64], "C": [200, 3, 130, 65],
-           "D": [140, 1, 5, 66]}
+           "D": [140, 1, 5, 66], "E": [170, 2, 64, 129]}
 # bfloat16 engine against the float64 oracle on these order-one weights: root-mean-square
 # error relative to the logits' root-mean-square, and largest error relative to the largest
 # logit (two norms a sublayer, a recurrent state and up to seven layer runs round more often

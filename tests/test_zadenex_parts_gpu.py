@@ -226,7 +226,11 @@ def plain_talking(params, mixer, x):
     talking_spec(n_heads=8, n_kv_heads=1, head_dim=8, value_dim=8, window=65),
     talking_spec(n_heads=2, n_kv_heads=2, head_dim=64, value_dim=64, window=None),
     talking_spec(n_heads=20, n_kv_heads=5, head_dim=16, value_dim=4, window=1),
-    talking_spec(n_heads=3, n_kv_heads=1, head_dim=40, value_dim=3, window=130)])
+    talking_spec(n_heads=3, n_kv_heads=1, head_dim=40, value_dim=3, window=130),
+    # sizes that the matrix-core kernel for wide keys takes in bfloat16: groups of 3, 4 and 1
+    talking_spec(n_heads=6, n_kv_heads=2, head_dim=16, value_dim=16, window=21),
+    talking_spec(n_heads=16, n_kv_heads=4, head_dim=32, value_dim=48, window=70),
+    talking_spec(n_heads=5, n_kv_heads=5, head_dim=32, value_dim=32, window=None)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_talking_attention_alone(mixer, dtype):
     """Whole, in portions and token by token, over the window's edge and two page borders."""
@@ -307,7 +311,11 @@ def plain_latent(params, mixer, x):
 @pytest.mark.parametrize("mixer", [
     latent_spec(), latent_spec(n_heads=1, head_dim=32, rot_dim=16, value_dim=40, kv_rank=24, q_rank=56),
     latent_spec(n_heads=20, head_dim=8, rot_dim=2, value_dim=8, kv_rank=72, q_rank=16, theta=500.0),
-    latent_spec(n_heads=5, head_dim=24, rot_dim=32, value_dim=12, kv_rank=264, q_rank=40, scale=0.1)])
+    latent_spec(n_heads=5, head_dim=24, rot_dim=32, value_dim=12, kv_rank=264, q_rank=40, scale=0.1),
+    # cache rows that the matrix-core kernel for wide keys takes in bfloat16; 3, 20 and 70 heads
+    latent_spec(kv_rank=48, rot_dim=16),
+    latent_spec(n_heads=20, head_dim=8, rot_dim=32, value_dim=8, kv_rank=96, q_rank=16),
+    latent_spec(n_heads=70, head_dim=8, rot_dim=32, value_dim=4, kv_rank=32, q_rank=32)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_latent_attention_alone(mixer, dtype):
     spec = one_layer(mixer)
@@ -315,6 +323,7 @@ def test_latent_attention_alone(mixer, dtype):
     params["layers.0.mixer.sink"][0] = 3.0          # a sink that outweighs the first keys
     model, session = session_for(spec, params, dtype)
     part = model.layers[0].mixer
+    assert part.wide == (dtype == "bfloat16" and mixer.cache_width % 32 == 0 and mixer.kv_rank % 16 == 0)
     torch.manual_seed(8)
     x = torch.randn(150, HIDDEN).to(torch.bfloat16).float()
     want = plain_latent(params, mixer, x.double())

@@ -67,7 +67,12 @@ CONFIG_C = model(150, 128, 1e-6, 0.7, 0.25, (0, 3, 2), [
 CONFIG_D = model(120, 48, 1e-5, 1.5, 0.8, (1, 2, 1), [
     latent(20, 8, 4, 8, 72, 16, 0.3, 20000.0, 64),
     attention(2, 1, 24, 40, 0.2, 3, 56)])
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D}
+# sizes that the matrix-core attention kernel for wide keys takes in bfloat16
+CONFIG_E = model(180, 64, 1e-6, 1.2, 0.6, (1, 3, 2), [
+    attention(8, 2, 16, 32, 0.25, 50, 96),
+    latent(4, 16, 16, 16, 48, 32, 0.2, 10000.0, 64),
+    mlstm(2, 16, 32, 12.0, 48)])
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D, "E": CONFIG_E}
 
 
 def tensor_shapes(cfg):
