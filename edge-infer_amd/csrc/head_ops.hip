@@ -75,21 +75,28 @@ __global__ void latent_down_store_kernel(
 
 constexpr int kTileRows = 16;
 constexpr int kTileK = 128;
+constexpr int kCols = 64;            // output columns of a block
+constexpr int kParts = 4;            // threads that share a column, each a quarter of a K tile
 
-// Block: head blockIdx.y, rows blockIdx.x * 16 .., output columns blockIdx.z * 256 + thread.
+// Block: head blockIdx.y, rows blockIdx.x * 16 .., output columns blockIdx.z * 64 + t % 64; the
+// four threads of a column take a quarter of every K tile each (eight weights requested at a
+// time, so that a step of few rows is not a chain of trips to memory) and add up through LDS.
 template <typename TI, typename TW, typename TO>
 __global__ void __launch_bounds__(256)
 head_matmul_kernel(const TI* __restrict__ x, int nsplit, size_t split_stride, long long x_row,
                    int x_head, int x_first, const TW* __restrict__ m, TO* __restrict__ y,
                    long long y_row, int y_head, int y_first, int N, int K, int J) {
   __shared__ float xs[kTileRows][kTileK];
+  __shared__ float sums[kParts][kTileRows][kCols];
   const int h = blockIdx.y;
   const int row0 = blockIdx.x * kTileRows;
-  const int j = blockIdx.z * 256 + threadIdx.x;
+  const int col = threadIdx.x % kCols, part = threadIdx.x / kCols;
+  const int j = blockIdx.z * kCols + col;
   const TW* mh = m + static_cast<size_t>(h) * K * J;
   float acc[kTileRows];
 #pragma unroll
   for (int r = 0; r < kTileRows; ++r) acc[r] = 0.f;
+  constexpr int kQuarter = kTileK / kParts;
   for (int k0 = 0; k0 < K; k0 += kTileK) {
     const int kn = min(kTileK, K - k0);
     __syncthreads();
@@ -103,19 +110,33 @@ head_matmul_kernel(const TI* __restrict__ x, int nsplit, size_t split_stride, lo
     }
     __syncthreads();
     if (j < J) {
-      for (int k = 0; k < kn; ++k) {
-        const float w = ei::to_f32<TW>(mh[static_cast<size_t>(k0 + k) * J + j]);
+      const int k_lo = part * kQuarter, k_hi = min(kn, k_lo + kQuarter);
+      for (int k = k_lo; k < k_hi; k += 8) {
+        float w[8];
 #pragma unroll
-        for (int r = 0; r < kTileRows; ++r) acc[r] += xs[r][k] * w;
+        for (int u = 0; u < 8; ++u)
+          w[u] = k + u < k_hi ? ei::to_f32<TW>(mh[static_cast<size_t>(k0 + k + u) * J + j]) : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (k + u < k_hi) {
+#pragma unroll
+            for (int r = 0; r < kTileRows; ++r) acc[r] += xs[r][k + u] * w[u];
+          }
+        }
       }
     }
   }
-  if (j < J) {
 #pragma unroll
-    for (int r = 0; r < kTileRows; ++r)
-      if (row0 + r < N)
-        y[static_cast<size_t>(row0 + r) * y_row + h * y_head + y_first + j] =
-            ei::from_f32<TO>(acc[r]);
+  for (int r = 0; r < kTileRows; ++r) sums[part][r][col] = acc[r];
+  __syncthreads();
+  // thread (part, col) finishes rows part, part + 4, ...
+  if (j < J) {
+    for (int r = part; r < kTileRows; r += kParts) {
+      if (row0 + r < N) {
+        const float total = (sums[0][r][col] + sums[1][r][col]) + (sums[2][r][col] + sums[3][r][col]);
+        y[static_cast<size_t>(row0 + r) * y_row + h * y_head + y_first + j] = ei::from_f32<TO>(total);
+      }
+    }
   }
 }
 
@@ -219,8 +240,9 @@ extern "C" int ei_head_matmul(const void* x, int x_dtype, int nsplit, long long 
                  static_cast<long long>(heads - 1) * x_head + x_first + K <= x_row &&
                  static_cast<long long>(heads - 1) * y_head + y_first + J <= y_row,
              "head_matmul: a head's part lies outside its row");
-  EI_REQUIRE(heads <= 65535 && (J + 255) / 256 <= 65535, "head_matmul: too many heads or columns");
-  dim3 grid((N + kTileRows - 1) / kTileRows, heads, (J + 255) / 256);
+  EI_REQUIRE(heads <= 65535 && (J + kCols - 1) / kCols <= 65535,
+             "head_matmul: too many heads or columns");
+  dim3 grid((N + kTileRows - 1) / kTileRows, heads, (J + kCols - 1) / kCols);
   const size_t ss = static_cast<size_t>(split_stride);
 #define EI_HM_CASE(TI, TW, TO)                                                                  \
   head_matmul_kernel<TI, TW, TO><<<grid, 256, 0, stream>>>(                                     \

@@ -9,22 +9,22 @@
 // The gates come from two columns a head of the fused projection: with a cap c,
 //   i_t = c tanh((x_i + b_i) / c),   f_t = logsigmoid(c tanh((x_f + b_f) / c)).
 //
-// `mlstm_walk`: a block per (sequence, head, block of columns of S) walks the sequence's rows
-// of the step in order.  A thread owns 8 neighbouring rows of one column of S in registers (and
-// the same rows of n); the L = key size / 8 lanes of a column add their partial dot products
-// with wave shuffles.  Tokens come through LDS in tiles of 16: q, k, the block's columns of v,
-// and the three factors of every token, which one thread works out in order (the only chain
-// besides S itself).  The state is read from one row of the table and written, whole, to
-// another (the table has two versions a sequence).
+// `mlstm_walk`: a block of one wave per (sequence, head, block of columns of S) walks the
+// sequence's rows of the step in order.  A thread owns 8 or 16 neighbouring rows of one column of
+// S in registers (and the same rows of n); the L lanes that share a column add their partial dot
+// products with DPP adds (a row swap for L = 32).  Tokens come through LDS in tiles of 16: q, k
+// (16 bytes a load where the projection is bfloat16), the block's columns of v, and the three
+// factors of every token, which one lane works out in order (the only chain besides S itself).
+// The state is read from one row of the table and written, whole, to another (the table has two
+// versions a sequence).
 // `mlstm_out`: a wave a (row, head): RMS norm of the read-out, a weight as wide as all heads,
 // a sigmoid gate from the projection, one rounding.
 #include "common.h"
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kOwn = 8;        // rows of a column that a thread owns
-constexpr int kTile = 16;      // tokens in LDS at a time
+constexpr int kThreads = EI_WAVE;   // a block is one wave
+constexpr int kTile = 16;           // tokens in LDS at a time
 
 template <typename TI>
 __device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_stride) {
@@ -35,6 +35,26 @@ __device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_st
 
 __device__ __forceinline__ float log_sigmoid(float z) {
   return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+}
+
+#define EI_DPP_ADD(v, ctrl)                                                                     \
+  ((v) + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (v)), \
+                                                                (ctrl), 0xf, 0xf, false)))
+
+// Sum over each aligned group of L neighbouring lanes (L a power of two up to 32), every lane
+// of the group getting it: quad permutes, mirrors of half rows and rows, a swap of
+// neighbouring rows.
+__device__ __forceinline__ float group_sum(float v, int L) {
+  if (L >= 2) v = EI_DPP_ADD(v, 0xb1);     // quad_perm [1,0,3,2]
+  if (L >= 4) v = EI_DPP_ADD(v, 0x4e);     // quad_perm [2,3,0,1]
+  if (L >= 8) v = EI_DPP_ADD(v, 0x141);    // row_half_mirror
+  if (L >= 16) v = EI_DPP_ADD(v, 0x140);   // row_mirror
+  if (L >= 32) {
+    const ei::ei_u32x2 r =
+        __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r.x) + __uint_as_float(r.y);
+  }
+  return v;
 }
 
 // Column offsets of the fused projection [q | k | v | i | f | g].
@@ -54,7 +74,7 @@ __host__ __device__ inline Columns columns_of(int heads, int dim, int vdim) {
   return c;
 }
 
-template <typename TI>
+template <typename TI, int OWN>
 __global__ void __launch_bounds__(kThreads)
 mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                   const float* __restrict__ i_bias, const float* __restrict__ f_bias,
@@ -64,7 +84,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                   float* __restrict__ o_raw, int heads, int dim, int vdim, int L, float cap,
                   float q_scale, float bottom_eps) {
   extern __shared__ float lds[];
-  const int dimP = L * kOwn;
+  const int dimP = L * OWN;
   const int CB = kThreads / L;                 // columns of S this block owns
   float* qs = lds;                             // [kTile][dimP]
   float* ks = qs + kTile * dimP;               // [kTile][dimP]
@@ -84,33 +104,56 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   const int t = threadIdx.x;
   const int part = t % L, col_local = t / L;
   const int col = blockIdx.y * CB + col_local;
-  const int r0 = part * kOwn;
+  const int r0 = part * OWN;
   const size_t head_floats = static_cast<size_t>(vdim) * dim + dim + 1;
   const float* in = state + static_cast<size_t>(seq_in[seq]) * state_stride + a * head_floats;
   float* out = state + static_cast<size_t>(seq_out[seq]) * state_stride + a * head_floats;
+  // 16-byte loads of q and k: a bfloat16 projection whose head parts start at multiples of 8
+  const bool octets = sizeof(TI) == 2 && nsplit == 1 && dim % 8 == 0 && P % 8 == 0;
 
-  float S[kOwn], nn[kOwn];
+  float S[OWN], nn[OWN];
 #pragma unroll
-  for (int r = 0; r < kOwn; ++r) {
+  for (int r = 0; r < OWN; ++r) {
     const bool live = r0 + r < dim;
     S[r] = (live && col < vdim) ? in[static_cast<size_t>(col) * dim + r0 + r] : 0.f;
     nn[r] = live ? in[static_cast<size_t>(vdim) * dim + r0 + r] : 0.f;
   }
-  float m_run = in[static_cast<size_t>(vdim) * dim + dim];      // used by thread 0 only
+  float m_run = in[static_cast<size_t>(vdim) * dim + dim];      // used by lane 0 only
 
   for (int t0 = 0; t0 < count; t0 += kTile) {
     const int tn = min(kTile, count - t0);
     __syncthreads();
-    for (int idx = t; idx < kTile * dimP; idx += kThreads) {
-      const int tt = idx / dimP, d = idx % dimP;
-      float qv = 0.f, kv = 0.f;
-      if (tt < tn && d < dim) {
-        const TI* src = proj + static_cast<size_t>(row0 + t0 + tt) * P + a * dim + d;
-        qv = sliced<TI>(src + col_of.q, nsplit, split_stride) * q_scale;
-        kv = sliced<TI>(src + col_of.k, nsplit, split_stride);
+    if (octets) {
+      const int per_row = dimP / 8;
+      for (int idx = t; idx < kTile * per_row; idx += kThreads) {
+        const int tt = idx / per_row, d = (idx % per_row) * 8;
+        float qv[8], kv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qv[e] = kv[e] = 0.f;
+        if (tt < tn && d < dim) {
+          const bf16_t* src = reinterpret_cast<const bf16_t*>(proj) +
+                              static_cast<size_t>(row0 + t0 + tt) * P + a * dim + d;
+          ei::VecN<bf16_t, 8>::load(src + col_of.q, qv);
+          ei::VecN<bf16_t, 8>::load(src + col_of.k, kv);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          qs[tt * dimP + d + e] = qv[e] * q_scale;
+          ks[tt * dimP + d + e] = kv[e];
+        }
       }
-      qs[idx] = qv;
-      ks[idx] = kv;
+    } else {
+      for (int idx = t; idx < kTile * dimP; idx += kThreads) {
+        const int tt = idx / dimP, d = idx % dimP;
+        float qv = 0.f, kv = 0.f;
+        if (tt < tn && d < dim) {
+          const TI* src = proj + static_cast<size_t>(row0 + t0 + tt) * P + a * dim + d;
+          qv = sliced<TI>(src + col_of.q, nsplit, split_stride) * q_scale;
+          kv = sliced<TI>(src + col_of.k, nsplit, split_stride);
+        }
+        qs[idx] = qv;
+        ks[idx] = kv;
+      }
     }
     for (int idx = t; idx < kTile * CB; idx += kThreads) {
       const int tt = idx / CB, c = blockIdx.y * CB + idx % CB;
@@ -139,24 +182,28 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
       }
     }
     __syncthreads();
+#pragma unroll 2
     for (int tt = 0; tt < tn; ++tt) {
       const float keep = keep_s[tt], take = take_s[tt];
       const float tv = take * vs[tt * CB + col_local];
       const float* kr = ks + tt * dimP + r0;
       const float* qr = qs + tt * dimP + r0;
+      float kk[OWN], qq[OWN];
+#pragma unroll
+      for (int r = 0; r < OWN; r += 4) {
+        ei::Vec4<float>::load(kr + r, *reinterpret_cast<float(*)[4]>(&kk[r]));
+        ei::Vec4<float>::load(qr + r, *reinterpret_cast<float(*)[4]>(&qq[r]));
+      }
       float dot_s = 0.f, dot_n = 0.f;
 #pragma unroll
-      for (int r = 0; r < kOwn; ++r) {
-        const float k = kr[r], q = qr[r];
-        S[r] = keep * S[r] + k * tv;
-        nn[r] = keep * nn[r] + take * k;
-        dot_s += S[r] * q;
-        dot_n += nn[r] * q;
+      for (int r = 0; r < OWN; ++r) {
+        S[r] = keep * S[r] + kk[r] * tv;
+        nn[r] = keep * nn[r] + take * kk[r];
+        dot_s += S[r] * qq[r];
+        dot_n += nn[r] * qq[r];
       }
-      for (int offset = L / 2; offset > 0; offset >>= 1) {
-        dot_s += __shfl_xor(dot_s, offset, EI_WAVE);
-        dot_n += __shfl_xor(dot_n, offset, EI_WAVE);
-      }
+      dot_s = group_sum(dot_s, L);
+      dot_n = group_sum(dot_n, L);
       if (part == 0 && col < vdim)
         o_raw[static_cast<size_t>(row0 + t0 + tt) * heads * vdim + a * vdim + col] =
             dot_s / (fmaxf(fabsf(dot_n), floor_s[tt]) + bottom_eps);
@@ -164,7 +211,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   }
 
 #pragma unroll
-  for (int r = 0; r < kOwn; ++r) {
+  for (int r = 0; r < OWN; ++r) {
     if (r0 + r < dim) {
       if (col < vdim) out[static_cast<size_t>(col) * dim + r0 + r] = S[r];
       if (blockIdx.y == 0 && col_local == 0) out[static_cast<size_t>(vdim) * dim + r0 + r] = nn[r];
@@ -199,9 +246,12 @@ __global__ void mlstm_out_kernel(const float* __restrict__ o_raw, const TI* __re
   }
 }
 
-int lanes_for(int dim) {
+// Rows of a column that a thread owns: 16 where that still leaves a column several lanes.
+int rows_owned(int dim) { return dim > 64 ? 16 : 8; }
+
+int lanes_for(int dim, int own) {
   int L = 1;
-  while (L * kOwn < dim) L *= 2;
+  while (L * own < dim) L *= 2;
   return L;
 }
 
@@ -233,25 +283,26 @@ extern "C" int ei_mlstm_walk(const void* proj, int dtype, int nsplit, long long 
              "mlstm_walk: null pointer");
   EI_REQUIRE(state_stride >= ei_mlstm_state_floats(heads, dim, vdim),
              "mlstm_walk: state rows too short");
-  const int L = lanes_for(dim);
+  const int own = rows_owned(dim);
+  const int L = lanes_for(dim, own);
   const int CB = kThreads / L;
-  const size_t lds = sizeof(float) * (2 * static_cast<size_t>(kTile) * L * kOwn +
+  const size_t lds = sizeof(float) * (2 * static_cast<size_t>(kTile) * L * own +
                                       static_cast<size_t>(kTile) * CB + 5 * kTile);
   EI_REQUIRE(static_cast<long long>(n_seqs) * heads <= 0x7fffffffLL, "mlstm_walk: too many blocks");
+  EI_REQUIRE((vdim + CB - 1) / CB <= 65535, "mlstm_walk: too many blocks of columns");
   dim3 grid(n_seqs * heads, (vdim + CB - 1) / CB);
   const size_t ss = static_cast<size_t>(split_stride);
-  if (dtype == EI_F32)
-    mlstm_walk_kernel<float><<<grid, kThreads, lds, stream>>>(
-        static_cast<const float*>(proj), nsplit, ss, i_bias, f_bias, state,
-        static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, heads, dim,
-        vdim, L, cap, q_scale, bottom_eps);
-  else if (dtype == EI_BF16)
-    mlstm_walk_kernel<bf16_t><<<grid, kThreads, lds, stream>>>(
-        static_cast<const bf16_t*>(proj), nsplit, ss, i_bias, f_bias, state,
-        static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, heads, dim,
-        vdim, L, cap, q_scale, bottom_eps);
-  else
-    EI_REQUIRE(false, "mlstm_walk: unknown dtype");
+#define EI_WALK(TI, OWN)                                                                       \
+  mlstm_walk_kernel<TI, OWN><<<grid, kThreads, lds, stream>>>(                                 \
+      static_cast<const TI*>(proj), nsplit, ss, i_bias, f_bias, state,                         \
+      static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, heads,   \
+      dim, vdim, L, cap, q_scale, bottom_eps)
+  if (dtype == EI_F32 && own == 8) EI_WALK(float, 8);
+  else if (dtype == EI_F32) EI_WALK(float, 16);
+  else if (dtype == EI_BF16 && own == 8) EI_WALK(bf16_t, 8);
+  else if (dtype == EI_BF16) EI_WALK(bf16_t, 16);
+  else EI_REQUIRE(false, "mlstm_walk: unknown dtype");
+#undef EI_WALK
   EI_LAUNCH_CHECK();
 }
 

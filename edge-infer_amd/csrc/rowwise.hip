@@ -690,6 +690,77 @@ __global__ void norm_add_norm_kernel(float* __restrict__ residual, const TD* __r
     out[base + i] = ei::from_f32<TO>((row_values[i] * inv2) * w_next[i]);
 }
 
+// The same for widths that are a multiple of 4: 16-byte accesses, the row kept in registers,
+// the slices' loads issued eight at a time (they are added in slice order).
+template <typename TD, typename TO, int CHUNKS>
+__global__ void norm_add_norm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                         int nsplit, size_t split_stride,
+                                         const float* __restrict__ w_after,
+                                         const float* __restrict__ w_next, float eps,
+                                         TO* __restrict__ out, int H) {
+  __shared__ float scratch[16];
+  const size_t base = static_cast<size_t>(blockIdx.x) * H;
+  const int quads = H / 4;
+  float wa[CHUNKS][4], wn[CHUNKS][4], r[CHUNKS][4], x[CHUNKS][4];
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) {
+      Vec4<float>::load(w_after + qd * 4, wa[k]);
+      Vec4<float>::load(w_next + qd * 4, wn[k]);
+      Vec4<float>::load(residual + base + qd * 4, r[k]);
+    }
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    x[k][0] = x[k][1] = x[k][2] = x[k][3] = 0.f;
+    if (qd < quads) {
+      const TD* d = delta + base + qd * 4;
+      for (int s0 = 0; s0 < nsplit; s0 += 8) {
+        float v[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) Vec4<TD>::load(d + (s0 + u) * split_stride, v[u]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < nsplit) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) x[k][i] += v[u][i];
+          }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sum += x[k][i] * x[k][i];
+    }
+  }
+  const float inv = 1.0f / sqrtf(ei::block_sum(sum, scratch) / static_cast<float>(H) + eps);
+  float sum2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        r[k][i] += (x[k][i] * inv) * wa[k][i];
+        sum2 += r[k][i] * r[k][i];
+      }
+      Vec4<float>::store(residual + base + qd * 4, r[k]);
+    }
+  }
+  const float inv2 = 1.0f / sqrtf(ei::block_sum(sum2, scratch) / static_cast<float>(H) + eps);
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) {
+      float y[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = (r[k][i] * inv2) * wn[k][i];
+      Vec4<TO>::store(out + base + qd * 4, y);
+    }
+  }
+}
+
 // out[r] = [a[r] | b[r]] in the storage type: two float32 streams side by side as the operand
 // of one product.
 template <typename TO>
@@ -732,15 +803,33 @@ extern "C" int ei_norm_add_norm(float* residual, const void* delta, int delta_dt
   const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 128);
   const size_t lds = static_cast<size_t>(H) * sizeof(float);
   const size_t ss = static_cast<size_t>(split_stride);
-#define EI_NAN_CASE(TD, TO)                                                                  \
-  norm_add_norm_kernel<TD, TO><<<N, threads, lds, stream>>>(                                 \
+  const bool vec = H % 4 == 0 && ss % 4 == 0;
+  const int quads = H / 4;
+  // few rows: up to 1024 threads a row, so that many loads are in flight; many rows: 256
+  const int most = N >= 512 && quads <= 4 * 256 ? 256 : 1024;
+  int vthreads = (quads + EI_WAVE - 1) / EI_WAVE * EI_WAVE;
+  if (vthreads > most) vthreads = most;
+  const int chunks = vec ? (quads + vthreads - 1) / vthreads : 0;
+#define EI_NAN_VEC(TD, TO, C)                                                                \
+  norm_add_norm_vec_kernel<TD, TO, C><<<N, vthreads, 0, stream>>>(                           \
       residual, static_cast<const TD*>(delta), nsplit, ss, w_after, w_next, eps,             \
       static_cast<TO*>(out), H)
+#define EI_NAN_CASE(TD, TO)                                                                  \
+  do {                                                                                       \
+    if (chunks == 1) EI_NAN_VEC(TD, TO, 1);                                                  \
+    else if (chunks == 2) EI_NAN_VEC(TD, TO, 2);                                             \
+    else if (chunks == 3 || chunks == 4) EI_NAN_VEC(TD, TO, 4);                              \
+    else                                                                                     \
+      norm_add_norm_kernel<TD, TO><<<N, threads, lds, stream>>>(                             \
+          residual, static_cast<const TD*>(delta), nsplit, ss, w_after, w_next, eps,         \
+          static_cast<TO*>(out), H);                                                         \
+  } while (0)
   if (delta_dtype == EI_F32 && out_dtype == EI_F32) EI_NAN_CASE(float, float);
   else if (delta_dtype == EI_F32 && out_dtype == EI_BF16) EI_NAN_CASE(float, bf16_t);
   else if (delta_dtype == EI_BF16 && out_dtype == EI_BF16) EI_NAN_CASE(bf16_t, bf16_t);
   else EI_REQUIRE(false, "norm_add_norm: unsupported dtype combination");
 #undef EI_NAN_CASE
+#undef EI_NAN_VEC
   EI_LAUNCH_CHECK();
 }
 
