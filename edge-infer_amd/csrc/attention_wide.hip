@@ -102,8 +102,10 @@ attn_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_page
       if (key0 + kKeys <= lo_key) continue;
       __syncthreads();
       // keys as stored; with values inside the keys, their first DV elements transposed as well
+      // (neighbouring lanes take neighbouring keys: their 2-byte writes of the transposed
+      // values then fall into 32 banks, two lanes a word, instead of into two banks)
       for (int ch = t; ch < kKeys * k_chunks; ch += kThreads) {
-        const int key = ch / k_chunks, col = (ch % k_chunks) * 8;
+        const int key = ch % kKeys, col = (ch / kKeys) * 8;
         const int kh = KH > 1 ? col / D : g, dd = KH > 1 ? col % D : col;
         uint4 val = uint4{0u, 0u, 0u, 0u};
         if (key0 + key <= hi_key)       // later slots hold stale bytes
@@ -121,7 +123,7 @@ attn_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_page
       }
       if (!values_in_keys) {
         for (int ch = t; ch < kKeys * v_chunks; ch += kThreads) {
-          const int key = ch / v_chunks, col = (ch % v_chunks) * 8;
+          const int key = ch % kKeys, col = (ch / kKeys) * 8;
           uint4 val = uint4{0u, 0u, 0u, 0u};
           if (key0 + key <= hi_key)
             val = *reinterpret_cast<const uint4*>(

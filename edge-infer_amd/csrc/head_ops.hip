@@ -79,8 +79,8 @@ constexpr int kCols = 64;            // output columns of a block
 constexpr int kParts = 4;            // threads that share a column, each a quarter of a K tile
 
 // Block: head blockIdx.y, rows blockIdx.x * 16 .., output columns blockIdx.z * 64 + t % 64; the
-// four threads of a column take a quarter of every K tile each (eight weights requested at a
-// time, so that a step of few rows is not a chain of trips to memory) and add up through LDS.
+// four threads of a column take a quarter of every K tile each (all its weights requested at
+// once, so that a step of few rows is not a chain of trips to memory) and add up through LDS.
 template <typename TI, typename TW, typename TO>
 __global__ void __launch_bounds__(256)
 head_matmul_kernel(const TI* __restrict__ x, int nsplit, size_t split_stride, long long x_row,
@@ -111,17 +111,16 @@ head_matmul_kernel(const TI* __restrict__ x, int nsplit, size_t split_stride, lo
     __syncthreads();
     if (j < J) {
       const int k_lo = part * kQuarter, k_hi = min(kn, k_lo + kQuarter);
-      for (int k = k_lo; k < k_hi; k += 8) {
-        float w[8];
+      // the thread's whole quarter of the tile is requested before any of it is used
+      float w[kQuarter];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          w[u] = k + u < k_hi ? ei::to_f32<TW>(mh[static_cast<size_t>(k0 + k + u) * J + j]) : 0.f;
+      for (int u = 0; u < kQuarter; ++u)
+        w[u] = k_lo + u < k_hi ? ei::to_f32<TW>(mh[static_cast<size_t>(k0 + k_lo + u) * J + j]) : 0.f;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          if (k + u < k_hi) {
+      for (int u = 0; u < kQuarter; ++u) {
+        if (k_lo + u < k_hi) {
 #pragma unroll
-            for (int r = 0; r < kTileRows; ++r) acc[r] += xs[r][k + u] * w[u];
-          }
+          for (int r = 0; r < kTileRows; ++r) acc[r] += xs[r][k_lo + u] * w[u];
         }
       }
     }

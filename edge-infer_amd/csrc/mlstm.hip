@@ -12,9 +12,11 @@
 // `mlstm_walk`: a block of one wave per (sequence, head, block of columns of S) walks the
 // sequence's rows of the step in order.  A thread owns 8 or 16 neighbouring rows of one column of
 // S in registers (and the same rows of n); the L lanes that share a column add their partial dot
-// products with DPP adds (a row swap for L = 32).  Tokens come through LDS in tiles of 16: q, k
+// products with DPP adds (a row swap for L = 32).  Tokens come through LDS in tiles of 32: q, k
 // (16 bytes a load where the projection is bfloat16), the block's columns of v, and the three
-// factors of every token, which one lane works out in order (the only chain besides S itself).
+// factors of every token.  A lane a token works those out: with F_t the sum of the tile's log
+// forget gates up to t, m_t = F_t + max(m before the tile, max over s <= t of (i_s - F_s)), a
+// prefix sum and a prefix maximum over the lanes, so nothing but S itself is a chain.
 // The state is read from one row of the table and written, whole, to another (the table has two
 // versions a sequence).
 // `mlstm_out`: a wave a (row, head): RMS norm of the read-out, a weight as wide as all heads,
@@ -24,7 +26,7 @@
 namespace {
 
 constexpr int kThreads = EI_WAVE;   // a block is one wave
-constexpr int kTile = 16;           // tokens in LDS at a time
+constexpr int kTile = 32;           // tokens in LDS at a time
 
 template <typename TI>
 __device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_stride) {
@@ -92,8 +94,6 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   float* keep_s = vs + kTile * CB;             // [kTile] e^(f + m' - m)
   float* take_s = keep_s + kTile;              // [kTile] e^(i - m)
   float* floor_s = take_s + kTile;             // [kTile] e^(-m)
-  float* gate_i = floor_s + kTile;             // [kTile] capped log input gate
-  float* gate_f = gate_i + kTile;              // [kTile] log forget gate
 
   const int seq = blockIdx.x / heads, a = blockIdx.x % heads;
   const int count = seq_count[seq];
@@ -118,7 +118,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
     S[r] = (live && col < vdim) ? in[static_cast<size_t>(col) * dim + r0 + r] : 0.f;
     nn[r] = live ? in[static_cast<size_t>(vdim) * dim + r0 + r] : 0.f;
   }
-  float m_run = in[static_cast<size_t>(vdim) * dim + dim];      // used by lane 0 only
+  float m_run = in[static_cast<size_t>(vdim) * dim + dim];
 
   for (int t0 = 0; t0 < count; t0 += kTile) {
     const int tn = min(kTile, count - t0);
@@ -163,23 +163,37 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                        nsplit, split_stride);
       vs[idx] = v;
     }
-    if (t < tn) {
-      const TI* src = proj + static_cast<size_t>(row0 + t0 + t) * P;
-      const float xi = sliced<TI>(src + col_of.i + a, nsplit, split_stride) + i_bias[a];
-      const float xf = sliced<TI>(src + col_of.f + a, nsplit, split_stride) + f_bias[a];
-      gate_i[t] = cap * tanhf(xi / cap);
-      gate_f[t] = log_sigmoid(cap * tanhf(xf / cap));
-    }
-    __syncthreads();
-    if (t == 0) {
-      for (int tt = 0; tt < tn; ++tt) {
-        const float li = gate_i[tt], lf = gate_f[tt];
-        const float m_new = fmaxf(lf + m_run, li);
-        keep_s[tt] = expf(lf + m_run - m_new);
-        take_s[tt] = expf(li - m_new);
-        floor_s[tt] = expf(-m_new);
-        m_run = m_new;
+    {
+      // lane t: token t of the tile (lanes beyond the tile's tokens carry neutral gates)
+      float li = -INFINITY, lf = 0.f;
+      if (t < tn) {
+        const TI* src = proj + static_cast<size_t>(row0 + t0 + t) * P;
+        const float xi = sliced<TI>(src + col_of.i + a, nsplit, split_stride) + i_bias[a];
+        const float xf = sliced<TI>(src + col_of.f + a, nsplit, split_stride) + f_bias[a];
+        li = cap * tanhf(xi / cap);
+        lf = log_sigmoid(cap * tanhf(xf / cap));
       }
+      float F = lf;                              // sum of the log forget gates up to this token
+#pragma unroll
+      for (int step = 1; step < kTile; step *= 2) {
+        const float other = __shfl_up(F, step, EI_WAVE);
+        if (t >= step) F += other;
+      }
+      float u = li - F;                          // largest i_s - F_s up to this token
+#pragma unroll
+      for (int step = 1; step < kTile; step *= 2) {
+        const float other = __shfl_up(u, step, EI_WAVE);
+        if (t >= step) u = fmaxf(u, other);
+      }
+      const float m_here = F + fmaxf(m_run, u);
+      float m_before = __shfl_up(m_here, 1, EI_WAVE);
+      if (t == 0) m_before = m_run;
+      if (t < tn) {
+        keep_s[t] = expf(lf + m_before - m_here);
+        take_s[t] = expf(li - m_here);
+        floor_s[t] = expf(-m_here);
+      }
+      m_run = __shfl(m_here, tn - 1, EI_WAVE);   // every lane carries the tile's last m
     }
     __syncthreads();
 #pragma unroll 2
@@ -287,7 +301,7 @@ extern "C" int ei_mlstm_walk(const void* proj, int dtype, int nsplit, long long 
   const int L = lanes_for(dim, own);
   const int CB = kThreads / L;
   const size_t lds = sizeof(float) * (2 * static_cast<size_t>(kTile) * L * own +
-                                      static_cast<size_t>(kTile) * CB + 5 * kTile);
+                                      static_cast<size_t>(kTile) * CB + 3 * kTile);
   EI_REQUIRE(static_cast<long long>(n_seqs) * heads <= 0x7fffffffLL, "mlstm_walk: too many blocks");
   EI_REQUIRE((vdim + CB - 1) / CB <= 65535, "mlstm_walk: too many blocks of columns");
   dim3 grid(n_seqs * heads, (vdim + CB - 1) / CB);

@@ -41,7 +41,9 @@ class LatentAttention:
 
     @property
     def capture_rows(self):
-        return min(self.down.capture_rows, self.up_q.capture_rows, self.o.capture_rows)
+        # (beyond the few-rows products' rows the per-head products are the library's as well)
+        return min(self.down.capture_rows, self.up_q.capture_rows, self.o.capture_rows,
+                   lib.SKINNY_ROWS)
 
     @classmethod
     def parameters(cls, spec, hidden):
@@ -149,6 +151,22 @@ class LatentAttention:
             wanted = (2 * self.compute_units + blocks - 1) // blocks
         return max(1, min(wanted, pages, MAX_SLICES))
 
+    def _per_head(self, ctx, x, matrices, y, x_head, x_first, y_head, y_first, name):
+        """y[n, h, y_first ..] = x[n, h, x_first ..] . matrices[h]: the library's batched product
+        for the many rows of a bfloat16 prompt step (as the framework's other products of many
+        rows), this package's kernel otherwise."""
+        heads, inner, outer = matrices.shape
+        rows = y.shape[0]
+        if self.dtype == torch.bfloat16 and rows > lib.SKINNY_ROWS and x.dim() == 2:
+            taken = x.view(rows, heads, x_head)[:, :, x_first:x_first + inner].transpose(0, 1)
+            made = ctx.buffer(name, (heads, rows, outer))
+            torch.bmm(taken, matrices, out=made)
+            y.view(rows, heads, y_head)[:, :, y_first:y_first + outer].copy_(made.transpose(0, 1))
+            ctx.release(made)
+        else:
+            lib.head_matmul(x, matrices, y, heads, x_head=x_head, x_first=x_first, y_head=y_head,
+                            y_first=y_first)
+
     def forward(self, ctx, x, entry):
         spec, meta = self.spec, ctx.meta
         H, d, r, rank = spec.n_heads, spec.head_dim, spec.rot_dim, spec.kv_rank
@@ -168,8 +186,7 @@ class LatentAttention:
         ctx.release(q_latent)
         # the queries in the latent's space: [W_uk^T q_plain | rotated q_turn] a head
         q_wide = ctx.buffer("latent.q_wide", (n, H * spec.cache_width))
-        lib.head_matmul(q, self.k_up, q_wide, H, x_head=d + r, x_first=0,
-                        y_head=spec.cache_width, y_first=0)
+        self._per_head(ctx, q, self.k_up, q_wide, d + r, 0, spec.cache_width, 0, "latent.q_made")
         if r:
             lib.rotate_pairs(q, self.frequencies, meta.row_pos, q_wide, H, r, x_head=d + r,
                              x_first=d, y_head=spec.cache_width, y_first=rank)
@@ -194,8 +211,7 @@ class LatentAttention:
                H, 1, spec.cache_width, **common)
         ctx.release(q_wide, gate, part_o, part_ml)
         out = ctx.buffer("latent.out", (n, spec.out_width))
-        lib.head_matmul(mixed, self.v_up, out, H, x_head=rank, x_first=0,
-                        y_head=spec.value_dim, y_first=0)
+        self._per_head(ctx, mixed, self.v_up, out, rank, 0, spec.value_dim, 0, "latent.v_made")
         ctx.release(mixed)
         delta = self.o.forward(ctx, out, "latent.o")
         ctx.release(out)
