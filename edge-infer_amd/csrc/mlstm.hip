@@ -10,9 +10,11 @@
 //   i_t = c tanh((x_i + b_i) / c),   f_t = logsigmoid(c tanh((x_f + b_f) / c)).
 //
 // `mlstm_walk`: a block of one wave per (sequence, head, block of columns of S) walks the
-// sequence's rows of the step in order.  A thread owns 8 or 16 neighbouring rows of one column of
-// S in registers (and the same rows of n); the L lanes that share a column add their partial dot
-// products with DPP adds (a row swap for L = 32).  Tokens come through LDS in tiles of 32: q, k
+// sequence's rows of the step in order.  A thread owns 8 neighbouring rows of four neighbouring
+// columns of S in registers (and the same rows of n, which all columns share: four independent
+// chains a thread, and k, q and n read and updated once for four columns); the L = key size / 8
+// lanes that share the columns add their partial dot products with DPP adds (a row swap for
+// L = 32).  Tokens come through LDS in tiles of 16: q, k
 // (16 bytes a load where the projection is bfloat16), the block's columns of v, and the three
 // factors of every token.  A lane a token works those out: with F_t the sum of the tile's log
 // forget gates up to t, m_t = F_t + max(m before the tile, max over s <= t of (i_s - F_s)), a
@@ -26,7 +28,9 @@
 namespace {
 
 constexpr int kThreads = EI_WAVE;   // a block is one wave
-constexpr int kTile = 32;           // tokens in LDS at a time
+constexpr int kTile = 16;           // tokens in LDS at a time
+constexpr int kOwn = 8;             // rows of a column that a thread owns
+constexpr int kCols = 4;            // columns of S that a thread owns
 
 template <typename TI>
 __device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_stride) {
@@ -76,7 +80,7 @@ __host__ __device__ inline Columns columns_of(int heads, int dim, int vdim) {
   return c;
 }
 
-template <typename TI, int OWN>
+template <typename TI>
 __global__ void __launch_bounds__(kThreads)
 mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                   const float* __restrict__ i_bias, const float* __restrict__ f_bias,
@@ -86,8 +90,9 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                   float* __restrict__ o_raw, int heads, int dim, int vdim, int L, float cap,
                   float q_scale, float bottom_eps) {
   extern __shared__ float lds[];
+  constexpr int OWN = kOwn, NC = kCols;
   const int dimP = L * OWN;
-  const int CB = kThreads / L;                 // columns of S this block owns
+  const int CB = kThreads / L * NC;            // columns of S this block owns
   float* qs = lds;                             // [kTile][dimP]
   float* ks = qs + kTile * dimP;               // [kTile][dimP]
   float* vs = ks + kTile * dimP;               // [kTile][CB]
@@ -102,8 +107,8 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   const Columns col_of = columns_of(heads, dim, vdim);
   const int P = col_of.width;
   const int t = threadIdx.x;
-  const int part = t % L, col_local = t / L;
-  const int col = blockIdx.y * CB + col_local;
+  const int part = t % L, group = t / L;
+  const int col0 = blockIdx.y * CB + group * NC;      // the thread's first column
   const int r0 = part * OWN;
   const size_t head_floats = static_cast<size_t>(vdim) * dim + dim + 1;
   const float* in = state + static_cast<size_t>(seq_in[seq]) * state_stride + a * head_floats;
@@ -111,11 +116,13 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   // 16-byte loads of q and k: a bfloat16 projection whose head parts start at multiples of 8
   const bool octets = sizeof(TI) == 2 && nsplit == 1 && dim % 8 == 0 && P % 8 == 0;
 
-  float S[OWN], nn[OWN];
+  float S[NC][OWN], nn[OWN];
 #pragma unroll
   for (int r = 0; r < OWN; ++r) {
     const bool live = r0 + r < dim;
-    S[r] = (live && col < vdim) ? in[static_cast<size_t>(col) * dim + r0 + r] : 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      S[c][r] = (live && col0 + c < vdim) ? in[static_cast<size_t>(col0 + c) * dim + r0 + r] : 0.f;
     nn[r] = live ? in[static_cast<size_t>(vdim) * dim + r0 + r] : 0.f;
   }
   float m_run = in[static_cast<size_t>(vdim) * dim + dim];
@@ -199,7 +206,10 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
 #pragma unroll 2
     for (int tt = 0; tt < tn; ++tt) {
       const float keep = keep_s[tt], take = take_s[tt];
-      const float tv = take * vs[tt * CB + col_local];
+      float tv[NC];
+      ei::Vec4<float>::load(vs + tt * CB + group * NC, tv);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) tv[c] *= take;
       const float* kr = ks + tt * dimP + r0;
       const float* qr = qs + tt * dimP + r0;
       float kk[OWN], qq[OWN];
@@ -208,27 +218,39 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
         ei::Vec4<float>::load(kr + r, *reinterpret_cast<float(*)[4]>(&kk[r]));
         ei::Vec4<float>::load(qr + r, *reinterpret_cast<float(*)[4]>(&qq[r]));
       }
-      float dot_s = 0.f, dot_n = 0.f;
+      float dot_s[NC], dot_n = 0.f;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) dot_s[c] = 0.f;
 #pragma unroll
       for (int r = 0; r < OWN; ++r) {
-        S[r] = keep * S[r] + kk[r] * tv;
         nn[r] = keep * nn[r] + take * kk[r];
-        dot_s += S[r] * qq[r];
         dot_n += nn[r] * qq[r];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          S[c][r] = keep * S[c][r] + kk[r] * tv[c];
+          dot_s[c] += S[c][r] * qq[r];
+        }
       }
-      dot_s = group_sum(dot_s, L);
       dot_n = group_sum(dot_n, L);
-      if (part == 0 && col < vdim)
-        o_raw[static_cast<size_t>(row0 + t0 + tt) * heads * vdim + a * vdim + col] =
-            dot_s / (fmaxf(fabsf(dot_n), floor_s[tt]) + bottom_eps);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) dot_s[c] = group_sum(dot_s[c], L);
+      if (part == 0) {
+        const float bottom = fmaxf(fabsf(dot_n), floor_s[tt]) + bottom_eps;
+        float* dst = o_raw + static_cast<size_t>(row0 + t0 + tt) * heads * vdim + a * vdim + col0;
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+          if (col0 + c < vdim) dst[c] = dot_s[c] / bottom;
+      }
     }
   }
 
 #pragma unroll
   for (int r = 0; r < OWN; ++r) {
     if (r0 + r < dim) {
-      if (col < vdim) out[static_cast<size_t>(col) * dim + r0 + r] = S[r];
-      if (blockIdx.y == 0 && col_local == 0) out[static_cast<size_t>(vdim) * dim + r0 + r] = nn[r];
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+        if (col0 + c < vdim) out[static_cast<size_t>(col0 + c) * dim + r0 + r] = S[c][r];
+      if (blockIdx.y == 0 && group == 0) out[static_cast<size_t>(vdim) * dim + r0 + r] = nn[r];
     }
   }
   if (blockIdx.y == 0 && t == 0) out[static_cast<size_t>(vdim) * dim + dim] = m_run;
@@ -260,12 +282,9 @@ __global__ void mlstm_out_kernel(const float* __restrict__ o_raw, const TI* __re
   }
 }
 
-// Rows of a column that a thread owns: 16 where that still leaves a column several lanes.
-int rows_owned(int dim) { return dim > 64 ? 16 : 8; }
-
-int lanes_for(int dim, int own) {
+int lanes_for(int dim) {
   int L = 1;
-  while (L * own < dim) L *= 2;
+  while (L * kOwn < dim) L *= 2;
   return L;
 }
 
@@ -297,24 +316,21 @@ extern "C" int ei_mlstm_walk(const void* proj, int dtype, int nsplit, long long 
              "mlstm_walk: null pointer");
   EI_REQUIRE(state_stride >= ei_mlstm_state_floats(heads, dim, vdim),
              "mlstm_walk: state rows too short");
-  const int own = rows_owned(dim);
-  const int L = lanes_for(dim, own);
-  const int CB = kThreads / L;
-  const size_t lds = sizeof(float) * (2 * static_cast<size_t>(kTile) * L * own +
+  const int L = lanes_for(dim);
+  const int CB = kThreads / L * kCols;
+  const size_t lds = sizeof(float) * (2 * static_cast<size_t>(kTile) * L * kOwn +
                                       static_cast<size_t>(kTile) * CB + 3 * kTile);
   EI_REQUIRE(static_cast<long long>(n_seqs) * heads <= 0x7fffffffLL, "mlstm_walk: too many blocks");
   EI_REQUIRE((vdim + CB - 1) / CB <= 65535, "mlstm_walk: too many blocks of columns");
   dim3 grid(n_seqs * heads, (vdim + CB - 1) / CB);
   const size_t ss = static_cast<size_t>(split_stride);
-#define EI_WALK(TI, OWN)                                                                       \
-  mlstm_walk_kernel<TI, OWN><<<grid, kThreads, lds, stream>>>(                                 \
+#define EI_WALK(TI)                                                                            \
+  mlstm_walk_kernel<TI><<<grid, kThreads, lds, stream>>>(                                      \
       static_cast<const TI*>(proj), nsplit, ss, i_bias, f_bias, state,                         \
       static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, heads,   \
       dim, vdim, L, cap, q_scale, bottom_eps)
-  if (dtype == EI_F32 && own == 8) EI_WALK(float, 8);
-  else if (dtype == EI_F32) EI_WALK(float, 16);
-  else if (dtype == EI_BF16 && own == 8) EI_WALK(bf16_t, 8);
-  else if (dtype == EI_BF16) EI_WALK(bf16_t, 16);
+  if (dtype == EI_F32) EI_WALK(float);
+  else if (dtype == EI_BF16) EI_WALK(bf16_t);
   else EI_REQUIRE(false, "mlstm_walk: unknown dtype");
 #undef EI_WALK
   EI_LAUNCH_CHECK();
