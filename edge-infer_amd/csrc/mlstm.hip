@@ -127,19 +127,79 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   }
   float m_run = in[static_cast<size_t>(vdim) * dim + dim];
 
+  // A long walk over a bfloat16 projection asks for a whole tile at once, from clamped places
+  // so that no load waits for a branch, and for the next tile while it walks this one.
+  constexpr int kAhead = 8;                    // most loads of a kind that a lane has in flight
+  const int per_row = dimP / 8;
+  const int qk_loads = (kTile * per_row + kThreads - 1) / kThreads;
+  const int v_loads = (kTile * CB + kThreads - 1) / kThreads;
+  const bool ahead = octets && qk_loads <= kAhead && v_loads <= kAhead;
+  const bf16_t* rows16 = reinterpret_cast<const bf16_t*>(proj);
+  uint4 q_pre[kAhead], k_pre[kAhead];
+  bf16_t v_pre[kAhead], xi_pre = 0, xf_pre = 0;
+  auto ask = [&](int t0) {
+    const int tn = min(kTile, count - t0);
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      if (i < qk_loads) {
+        const int idx = t + i * kThreads;
+        const int tt = min(idx / per_row, tn - 1), d = min((idx % per_row) * 8, dim - 8);
+        const bf16_t* src = rows16 + static_cast<size_t>(row0 + t0 + tt) * P + a * dim + d;
+        q_pre[i] = *reinterpret_cast<const uint4*>(src + col_of.q);
+        k_pre[i] = *reinterpret_cast<const uint4*>(src + col_of.k);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      if (i < v_loads) {
+        const int idx = t + i * kThreads;
+        const int tt = min(idx / CB, tn - 1), c = min(blockIdx.y * CB + idx % CB, vdim - 1);
+        v_pre[i] = rows16[static_cast<size_t>(row0 + t0 + tt) * P + col_of.v + a * vdim + c];
+      }
+    }
+    const bf16_t* gates = rows16 + static_cast<size_t>(row0 + t0 + min(t, tn - 1)) * P;
+    xi_pre = gates[col_of.i + a];
+    xf_pre = gates[col_of.f + a];
+  };
+  if (ahead) ask(0);
+
   for (int t0 = 0; t0 < count; t0 += kTile) {
     const int tn = min(kTile, count - t0);
     __syncthreads();
-    if (octets) {
-      const int per_row = dimP / 8;
+    if (ahead) {
+#pragma unroll
+      for (int i = 0; i < kAhead; ++i) {
+        const int idx = t + i * kThreads;
+        if (i < qk_loads && idx < kTile * per_row) {
+          const int tt = idx / per_row, d = (idx % per_row) * 8;
+          const bool live = tt < tn && d < dim;
+          const uint32_t qw[4] = {q_pre[i].x, q_pre[i].y, q_pre[i].z, q_pre[i].w};
+          const uint32_t kw[4] = {k_pre[i].x, k_pre[i].y, k_pre[i].z, k_pre[i].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            qs[tt * dimP + d + 2 * e] = live ? __uint_as_float(qw[e] << 16) * q_scale : 0.f;
+            qs[tt * dimP + d + 2 * e + 1] = live ? __uint_as_float(qw[e] & 0xffff0000u) * q_scale : 0.f;
+            ks[tt * dimP + d + 2 * e] = live ? __uint_as_float(kw[e] << 16) : 0.f;
+            ks[tt * dimP + d + 2 * e + 1] = live ? __uint_as_float(kw[e] & 0xffff0000u) : 0.f;
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kAhead; ++i) {
+        const int idx = t + i * kThreads;
+        if (i < v_loads && idx < kTile * CB) {
+          const bool live = idx / CB < tn && blockIdx.y * CB + idx % CB < vdim;
+          vs[idx] = live ? ei::bf16_to_f32(v_pre[i]) : 0.f;
+        }
+      }
+    } else if (octets) {
       for (int idx = t; idx < kTile * per_row; idx += kThreads) {
         const int tt = idx / per_row, d = (idx % per_row) * 8;
         float qv[8], kv[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) qv[e] = kv[e] = 0.f;
         if (tt < tn && d < dim) {
-          const bf16_t* src = reinterpret_cast<const bf16_t*>(proj) +
-                              static_cast<size_t>(row0 + t0 + tt) * P + a * dim + d;
+          const bf16_t* src = rows16 + static_cast<size_t>(row0 + t0 + tt) * P + a * dim + d;
           ei::VecN<bf16_t, 8>::load(src + col_of.q, qv);
           ei::VecN<bf16_t, 8>::load(src + col_of.k, kv);
         }
@@ -162,24 +222,36 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
         ks[idx] = kv;
       }
     }
-    for (int idx = t; idx < kTile * CB; idx += kThreads) {
-      const int tt = idx / CB, c = blockIdx.y * CB + idx % CB;
-      float v = 0.f;
-      if (tt < tn && c < vdim)
-        v = sliced<TI>(proj + static_cast<size_t>(row0 + t0 + tt) * P + col_of.v + a * vdim + c,
-                       nsplit, split_stride);
-      vs[idx] = v;
+    if (!ahead) {
+      for (int idx = t; idx < kTile * CB; idx += kThreads) {
+        const int tt = idx / CB, c = blockIdx.y * CB + idx % CB;
+        float v = 0.f;
+        if (tt < tn && c < vdim)
+          v = sliced<TI>(proj + static_cast<size_t>(row0 + t0 + tt) * P + col_of.v + a * vdim + c,
+                         nsplit, split_stride);
+        vs[idx] = v;
+      }
     }
     {
       // lane t: token t of the tile (lanes beyond the tile's tokens carry neutral gates)
       float li = -INFINITY, lf = 0.f;
       if (t < tn) {
-        const TI* src = proj + static_cast<size_t>(row0 + t0 + t) * P;
-        const float xi = sliced<TI>(src + col_of.i + a, nsplit, split_stride) + i_bias[a];
-        const float xf = sliced<TI>(src + col_of.f + a, nsplit, split_stride) + f_bias[a];
+        float xi, xf;
+        if (ahead) {
+          xi = ei::bf16_to_f32(xi_pre);
+          xf = ei::bf16_to_f32(xf_pre);
+        } else {
+          const TI* src = proj + static_cast<size_t>(row0 + t0 + t) * P;
+          xi = sliced<TI>(src + col_of.i + a, nsplit, split_stride);
+          xf = sliced<TI>(src + col_of.f + a, nsplit, split_stride);
+        }
+        xi += i_bias[a];
+        xf += f_bias[a];
         li = cap * tanhf(xi / cap);
         lf = log_sigmoid(cap * tanhf(xf / cap));
       }
+      // the next tile's loads travel while this one is walked
+      if (ahead && t0 + kTile < count) ask(t0 + kTile);
       float F = lf;                              // sum of the log forget gates up to this token
 #pragma unroll
       for (int step = 1; step < kTile; step *= 2) {
@@ -203,7 +275,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
       m_run = __shfl(m_here, tn - 1, EI_WAVE);   // every lane carries the tile's last m
     }
     __syncthreads();
-#pragma unroll 2
+#pragma unroll 4
     for (int tt = 0; tt < tn; ++tt) {
       const float keep = keep_s[tt], take = take_s[tt];
       float tv[NC];
@@ -235,11 +307,12 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
 #pragma unroll
       for (int c = 0; c < NC; ++c) dot_s[c] = group_sum(dot_s[c], L);
       if (part == 0) {
-        const float bottom = fmaxf(fabsf(dot_n), floor_s[tt]) + bottom_eps;
+        // (one division a token: the columns share the denominator)
+        const float over = 1.0f / (fmaxf(fabsf(dot_n), floor_s[tt]) + bottom_eps);
         float* dst = o_raw + static_cast<size_t>(row0 + t0 + tt) * heads * vdim + a * vdim + col0;
 #pragma unroll
         for (int c = 0; c < NC; ++c)
-          if (col0 + c < vdim) dst[c] = dot_s[c] / bottom;
+          if (col0 + c < vdim) dst[c] = dot_s[c] * over;
       }
     }
   }
