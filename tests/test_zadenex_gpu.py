@@ -15,9 +15,9 @@ from zadenex_helpers import CONFIGS, ids, sharp_weights, tensor_shapes, write_fo
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-NAMES = ["A", "B", "C", "D", "E"]
+NAMES = ["A", "B", "C", "D", "E", "F"]
 LENGTHS = {"A": [150, 1, 49, 75], "B": [210, 2, 101, 64], "C": [200, 3, 130, 65],
-           "D": [140, 1, 5, 66], "E": [170, 2, 64, 129]}
+           "D": [140, 1, 5, 66], "E": [170, 2, 64, 129], "F": [90, 1, 65, 8]}
 # bfloat16 engine against the float64 oracle on these order-one weights: root-mean-square
 # error relative to the logits' root-mean-square, and largest error relative to the largest
 # logit (two norms a sublayer, a recurrent state and up to seven layer runs round more often
@@ -209,7 +209,10 @@ def test_long_decoding_from_the_first_token(models, weights, name, dtype):
     slot = session.begin()
     rows = [session.step([(slot, [token], [0])]) for token in request]
     close(dtype, torch.cat(rows), ref, f"{name} {dtype} 300 tokens one by one")
-    assert session.graphs and session.graph_replays > 250
+    if session.graphs:     # (F in bfloat16 has products of odd widths, which the library multiplies)
+        assert session.graph_replays > 250
+    else:
+        assert (name, dtype) == ("F", "bfloat16")
 
 
 @pytest.mark.parametrize("graphs", [True, False])

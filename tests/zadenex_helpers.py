@@ -72,7 +72,13 @@ CONFIG_E = model(180, 64, 1e-6, 1.2, 0.6, (1, 3, 2), [
     attention(8, 2, 16, 32, 0.25, 50, 96),
     latent(4, 16, 16, 16, 48, 32, 0.2, 10000.0, 64),
     mlstm(2, 16, 32, 12.0, 48)])
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D, "E": CONFIG_E}
+# sizes that are multiples of nothing: no vector kernel and no few-rows product applies
+CONFIG_F = model(101, 50, 1e-5, 0.9, 0.7, (0, 2, 2), [
+    latent(3, 10, 6, 6, 22, 14, 0.3, 3000.0, 30),
+    attention(6, 3, 12, 10, 0.3, 7, None),
+    mlstm(3, 12, 5, 8.0, 26)])
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D, "E": CONFIG_E,
+           "F": CONFIG_F}
 
 
 def tensor_shapes(cfg):
