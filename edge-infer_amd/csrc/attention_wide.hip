@@ -232,6 +232,7 @@ attn_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_page
 }
 
 // One wave per (row, head): o = sum_s o_s e^{m_s - m} / sum_s l_s e^{m_s - m}, times the gate.
+// Lane s works out slice s's weight once (at most 64 slices); the lanes then share them.
 __global__ void wide_merge_kernel(const float* __restrict__ part_o,
                                   const float* __restrict__ part_ml,
                                   const int32_t* __restrict__ row_seq, bf16_t* __restrict__ out,
@@ -243,17 +244,25 @@ __global__ void wide_merge_kernel(const float* __restrict__ part_o,
   const int row = wave / nq;
   if (row_seq && row_seq[row] < 0) return;
   const float* ml = part_ml + static_cast<size_t>(wave) * n_splits * 2;
-  float m = kLowest;
-  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
-  float l = 0.f;
-  for (int s = 0; s < n_splits; ++s) l += ml[2 * s + 1] * expf(ml[2 * s] - m);
+  const float m_own = lane < n_splits ? ml[2 * lane] : kLowest;
+  const float l_own = lane < n_splits ? ml[2 * lane + 1] : 0.f;
+  const float m = ei::wave_max(m_own);
+  float weight = lane < n_splits ? expf(m_own - m) : 0.f;
+  const float l = ei::wave_sum(l_own * weight);
   float inv = l > 0.f ? 1.f / l : 0.f;
   if (gate) inv *= 1.0f / (1.0f + expf(-gate[wave]));
+  weight *= inv;
   const float* po = part_o + static_cast<size_t>(wave) * n_splits * DV;
-  for (int d = lane; d < DV; d += EI_WAVE) {
-    float o = 0.f;
-    for (int s = 0; s < n_splits; ++s) o += po[static_cast<size_t>(s) * DV + d] * expf(ml[2 * s] - m);
-    out[static_cast<size_t>(wave) * DV + d] = ei::from_f32<bf16_t>(o * inv);
+  for (int d = lane * 4; d < DV; d += EI_WAVE * 4) {       // DV is a multiple of 16
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < n_splits; ++s) {
+      float x[4];
+      ei::Vec4<float>::load(po + static_cast<size_t>(s) * DV + d, x);
+      const float w = __shfl(weight, s, EI_WAVE);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] += x[e] * w;
+    }
+    ei::Vec4<bf16_t>::store(out + static_cast<size_t>(wave) * DV + d, o);
   }
 }
 

@@ -29,7 +29,7 @@ _SIGNATURES = {
         "ei_add_rmsnorm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
                            c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int, c_int,
-                      c_int, c_void_p],
+                      c_int, c_void_p, c_void_p],
         "ei_norm_add_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
                              c_float, c_void_p, c_int, c_int, c_int, c_void_p],
         "ei_concat_cast": [c_void_p, c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
@@ -306,19 +306,23 @@ GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor, strip: int = 0,
-           activation: str = "silu") -> None:
+           activation: str = "silu", bias: Optional[torch.Tensor] = None) -> None:
     """out = act(gate) * up of [n, 2*inter] rows (or float32 slices of them), act "silu" or
     "gelu_tanh".  strip = 0: the gate columns come first, then the up columns; strip > 0:
-    `strip` gate columns, their `strip` up columns, and so on."""
+    `strip` gate columns, their `strip` up columns, and so on.  bias: float32 [2*inter] in the
+    rows' own column order, added before the activation."""
     lib = library("rowwise")
     if activation not in GATE_ACTIVATIONS:
         raise KernelError(f"swiglu: unknown gate activation '{activation}'; "
                           f"known: {sorted(GATE_ACTIVATIONS)}")
     n, inter = out.shape
     nsplit, stride = _splits(gate_up, n, 2 * inter, "gate_up")
+    if bias is not None and bias.numel() != 2 * inter:
+        raise KernelError("swiglu: the bias must be as wide as a row of gate_up")
     status = lib.ei_swiglu(_gpu(gate_up, "gate_up"), _code(gate_up, "gate_up"), nsplit, stride,
                            _gpu(out, "out"), _code(out, "out"), n, inter, int(strip),
-                           GATE_ACTIVATIONS[activation], _stream())
+                           GATE_ACTIVATIONS[activation],
+                           None if bias is None else _gpu(bias, "bias", torch.float32), _stream())
     _check(lib, status, "swiglu")
 
 

@@ -10,11 +10,13 @@
 //   i_t = c tanh((x_i + b_i) / c),   f_t = logsigmoid(c tanh((x_f + b_f) / c)).
 //
 // `mlstm_walk`: a block of one wave per (sequence, head, block of columns of S) walks the
-// sequence's rows of the step in order.  A thread owns 8 neighbouring rows of four neighbouring
-// columns of S in registers (and the same rows of n, which all columns share: four independent
-// chains a thread, and k, q and n read and updated once for four columns); the L = key size / 8
-// lanes that share the columns add their partial dot products with DPP adds (a row swap for
-// L = 32).  Tokens come through LDS in tiles of 16: q, k
+// sequence's rows of the step in order.  A thread owns 8 neighbouring rows of one, two or four
+// neighbouring columns of S in registers (and the same rows of n, which all its columns share);
+// the L = key size / 8 lanes that share the columns add their partial dot products with DPP
+// adds (a row swap for L = 32).  A wave that is alone on its SIMD pays for every instruction of
+// a token in full, so a launch of few blocks takes one column a thread (the fewest instructions
+// a token); where the chip is full anyway, four columns a thread read and update k, q and n
+// once for four columns (the fewest instructions in all).  Tokens come through LDS in tiles of 16: q, k
 // (16 bytes a load where the projection is bfloat16), the block's columns of v, and the three
 // factors of every token.  A lane a token works those out: with F_t the sum of the tile's log
 // forget gates up to t, m_t = F_t + max(m before the tile, max over s <= t of (i_s - F_s)), a
@@ -30,7 +32,7 @@ namespace {
 constexpr int kThreads = EI_WAVE;   // a block is one wave
 constexpr int kTile = 16;           // tokens in LDS at a time
 constexpr int kOwn = 8;             // rows of a column that a thread owns
-constexpr int kCols = 4;            // columns of S that a thread owns
+constexpr int kMostCols = 4;        // most columns of S that a thread owns (1, 2 or 4)
 
 template <typename TI>
 __device__ __forceinline__ float sliced(const TI* p, int nsplit, size_t split_stride) {
@@ -80,7 +82,7 @@ __host__ __device__ inline Columns columns_of(int heads, int dim, int vdim) {
   return c;
 }
 
-template <typename TI>
+template <typename TI, int NC>
 __global__ void __launch_bounds__(kThreads)
 mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                   const float* __restrict__ i_bias, const float* __restrict__ f_bias,
@@ -90,7 +92,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                   float* __restrict__ o_raw, int heads, int dim, int vdim, int L, float cap,
                   float q_scale, float bottom_eps) {
   extern __shared__ float lds[];
-  constexpr int OWN = kOwn, NC = kCols;
+  constexpr int OWN = kOwn;
   const int dimP = L * OWN;
   const int CB = kThreads / L * NC;            // columns of S this block owns
   float* qs = lds;                             // [kTile][dimP]
@@ -279,9 +281,8 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
     for (int tt = 0; tt < tn; ++tt) {
       const float keep = keep_s[tt], take = take_s[tt];
       float tv[NC];
-      ei::Vec4<float>::load(vs + tt * CB + group * NC, tv);
 #pragma unroll
-      for (int c = 0; c < NC; ++c) tv[c] *= take;
+      for (int c = 0; c < NC; ++c) tv[c] = take * vs[tt * CB + group * NC + c];
       const float* kr = ks + tt * dimP + r0;
       const float* qr = qs + tt * dimP + r0;
       float kk[OWN], qq[OWN];
@@ -390,21 +391,34 @@ extern "C" int ei_mlstm_walk(const void* proj, int dtype, int nsplit, long long 
   EI_REQUIRE(state_stride >= ei_mlstm_state_floats(heads, dim, vdim),
              "mlstm_walk: state rows too short");
   const int L = lanes_for(dim);
-  const int CB = kThreads / L * kCols;
+  // columns a thread: as many (4, 2, 1) as still give every SIMD of the chip two waves
+  const long long wanted = 2LL * 4 * ei_compute_units();
+  int nc = kMostCols;
+  while (nc > 1 && static_cast<long long>(n_seqs) * heads *
+                           ((vdim + kThreads / L * nc - 1) / (kThreads / L * nc)) < wanted)
+    nc /= 2;
+  const int CB = kThreads / L * nc;
   const size_t lds = sizeof(float) * (2 * static_cast<size_t>(kTile) * L * kOwn +
                                       static_cast<size_t>(kTile) * CB + 3 * kTile);
   EI_REQUIRE(static_cast<long long>(n_seqs) * heads <= 0x7fffffffLL, "mlstm_walk: too many blocks");
   EI_REQUIRE((vdim + CB - 1) / CB <= 65535, "mlstm_walk: too many blocks of columns");
   dim3 grid(n_seqs * heads, (vdim + CB - 1) / CB);
   const size_t ss = static_cast<size_t>(split_stride);
-#define EI_WALK(TI)                                                                            \
-  mlstm_walk_kernel<TI><<<grid, kThreads, lds, stream>>>(                                      \
+#define EI_WALK(TI, NC)                                                                        \
+  mlstm_walk_kernel<TI, NC><<<grid, kThreads, lds, stream>>>(                                  \
       static_cast<const TI*>(proj), nsplit, ss, i_bias, f_bias, state,                         \
       static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, heads,   \
       dim, vdim, L, cap, q_scale, bottom_eps)
-  if (dtype == EI_F32) EI_WALK(float);
-  else if (dtype == EI_BF16) EI_WALK(bf16_t);
+#define EI_WALK_COLS(TI)              \
+  do {                                \
+    if (nc == 4) EI_WALK(TI, 4);      \
+    else if (nc == 2) EI_WALK(TI, 2); \
+    else EI_WALK(TI, 1);              \
+  } while (0)
+  if (dtype == EI_F32) EI_WALK_COLS(float);
+  else if (dtype == EI_BF16) EI_WALK_COLS(bf16_t);
   else EI_REQUIRE(false, "mlstm_walk: unknown dtype");
+#undef EI_WALK_COLS
 #undef EI_WALK
   EI_LAUNCH_CHECK();
 }

@@ -149,7 +149,8 @@ __device__ __forceinline__ size_t gate_column(size_t col, int strip) {
 
 template <typename TI, typename TO>
 __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
-                              TO* __restrict__ out, int I, size_t total, int strip, int act) {
+                              TO* __restrict__ out, int I, size_t total, int strip, int act,
+                              const float* __restrict__ bias) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   const size_t up_offset = strip ? strip : I;
@@ -161,6 +162,10 @@ __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t
       gate += ei::to_f32<TI>(g[s * split_stride]);
       up += ei::to_f32<TI>(g[s * split_stride + up_offset]);
     }
+    if (bias) {        // laid out as a row of gate_up
+      gate += bias[gate_column(col, strip)];
+      up += bias[gate_column(col, strip) + up_offset];
+    }
     out[idx] = ei::from_f32<TO>(gate_act<TO>(gate, act) * up);
   }
 }
@@ -169,7 +174,8 @@ __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t
 // 16-byte (bfloat16) or 2 x 16-byte (float32) accesses.
 template <typename TI, typename TO>
 __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
-                                  TO* __restrict__ out, int I, size_t total_octets, int strip, int act) {
+                                  TO* __restrict__ out, int I, size_t total_octets, int strip, int act,
+                                  const float* __restrict__ bias) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   const int octets_per_row = I / 8;
@@ -203,6 +209,14 @@ __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, si
             up[i + 4] += d[u][i];
           }
         }
+    }
+    if (bias) {        // laid out as a row of gate_up
+      const float* b = bias + gate_column(col, strip);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        gate[i] += b[i];
+        up[i] += b[up_offset + i];
+      }
     }
     float y0[4], y1[4];
 #pragma unroll
@@ -355,7 +369,7 @@ extern "C" int ei_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
 // strip > 0 (a divisor of I): `strip` gate columns, their `strip` up columns, and so on.
 extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long long split_stride,
                          void* out, int out_dtype, int N, int I, int strip, int act,
-                         hipStream_t stream) {
+                         const float* bias, hipStream_t stream) {
   EI_REQUIRE(N > 0 && I > 0 && nsplit >= 1, "swiglu: sizes must be positive");
   EI_REQUIRE(act == 0 || act == 1, "swiglu: unknown gate activation");
   EI_REQUIRE(gate_up && out, "swiglu: null pointer");
@@ -369,13 +383,13 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
     if (vblocks > ei_compute_units() * 32) vblocks = ei_compute_units() * 32;
     if (in_dtype == EI_F32 && out_dtype == EI_F32)
       swiglu_vec_kernel<float, float><<<vblocks, threads, 0, stream>>>(
-          static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets, strip, act);
+          static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets, strip, act, bias);
     else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
       swiglu_vec_kernel<float, bf16_t><<<vblocks, threads, 0, stream>>>(
-          static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act);
+          static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act, bias);
     else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
       swiglu_vec_kernel<bf16_t, bf16_t><<<vblocks, threads, 0, stream>>>(
-          static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act);
+          static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip, act, bias);
     else
       EI_REQUIRE(false, "swiglu: unsupported dtype combination");
     EI_LAUNCH_CHECK();
@@ -384,13 +398,13 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
   if (blocks > ei_compute_units() * 32) blocks = ei_compute_units() * 32;
   if (in_dtype == EI_F32 && out_dtype == EI_F32)
     swiglu_kernel<float, float><<<blocks, threads, 0, stream>>>(
-        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total, strip, act);
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total, strip, act, bias);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
     swiglu_kernel<float, bf16_t><<<blocks, threads, 0, stream>>>(
-        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act);
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act, bias);
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
     swiglu_kernel<bf16_t, bf16_t><<<blocks, threads, 0, stream>>>(
-        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act);
+        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip, act, bias);
   else
     EI_REQUIRE(false, "swiglu: unsupported dtype combination");
   EI_LAUNCH_CHECK();

@@ -84,9 +84,10 @@ class GatedMLP:
         act = (self.gate_up.forward_gated(ctx, x, "mlp.act")
                if self.strip and self.spec.activation == "silu" else None)
         if act is None:
-            gate_up = self.gate_up.forward(ctx, x, "mlp.gate_up")
+            # (the activation kernel adds the bias itself where the product left it to it)
+            gate_up, bias = self.gate_up.forward(ctx, x, "mlp.gate_up", bias_later=True)
             act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
-            lib.swiglu(gate_up, act, self.strip, self.spec.activation)
+            lib.swiglu(gate_up, act, self.strip, self.spec.activation, bias=bias)
             ctx.release(gate_up)
         out = self.down.forward(ctx, act, "mlp.down")
         ctx.release(act)
