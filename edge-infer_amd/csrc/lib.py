@@ -31,14 +31,14 @@ _SIGNATURES = {
         "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int, c_int,
                       c_int, c_void_p, c_void_p],
         "ei_norm_add_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
-                             c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+                             c_float, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
         "ei_concat_cast": [c_void_p, c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
         "ei_set_rows": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_longlong, c_int,
                         c_void_p],
         "ei_sum_slices": [c_void_p, c_int, c_longlong, c_void_p, c_longlong, c_void_p],
         "ei_bias_rows": [c_void_p, c_void_p, c_longlong, c_int, c_int, c_void_p],
         "ei_norm_add": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_float, c_void_p,
-                        c_int, c_int, c_int, c_void_p],
+                        c_int, c_int, c_int, c_void_p, c_void_p],
         "ei_cast_rows": [c_void_p, c_void_p, c_int, c_longlong, c_void_p],
         "ei_activation": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_longlong, c_int,
                           c_void_p],
@@ -347,10 +347,18 @@ def bias_rows(bias: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
     _check(lib, status, "bias_rows")
 
 
+def _row_bias(bias, hidden, what):
+    if bias is None:
+        return None
+    if bias.numel() != hidden:
+        raise KernelError(f"{what}: the bias must have {hidden} elements")
+    return _gpu(bias, "bias", torch.float32)
+
+
 def norm_add(residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float,
-             cast_out: Optional[torch.Tensor] = None) -> None:
-    """residual [R, H] float32 += rmsnorm(sum of delta's slices) * weight; `cast_out` [R, H]
-    (optional) receives the new residual rows in its own type."""
+             cast_out: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> None:
+    """residual [R, H] float32 += rmsnorm(sum of delta's slices (+ bias [H])) * weight;
+    `cast_out` [R, H] (optional) receives the new residual rows in its own type."""
     lib = library("rowwise")
     rows, hidden = residual.shape
     nsplit, stride = _splits(delta, rows, hidden, "delta")
@@ -363,13 +371,14 @@ def norm_add(residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, 
                              _gpu(weight, "weight", torch.float32), float(eps),
                              None if cast_out is None else _gpu(cast_out, "cast_out"),
                              F32 if cast_out is None else _code(cast_out, "cast_out"), rows, hidden,
-                             _stream())
+                             _row_bias(bias, hidden, "norm_add"), _stream())
     _check(lib, status, "norm_add")
 
 
 def norm_add_norm(residual: torch.Tensor, delta: torch.Tensor, w_after: torch.Tensor,
-                  w_next: torch.Tensor, eps: float, out: torch.Tensor) -> None:
-    """residual [R, H] float32 += rmsnorm(sum of delta's slices) * w_after, then
+                  w_next: torch.Tensor, eps: float, out: torch.Tensor,
+                  bias: Optional[torch.Tensor] = None) -> None:
+    """residual [R, H] float32 += rmsnorm(sum of delta's slices (+ bias [H])) * w_after, then
     out [R, H] = rmsnorm(residual) * w_next in out's type: one pass over the rows."""
     lib = library("rowwise")
     rows, hidden = residual.shape
@@ -382,7 +391,8 @@ def norm_add_norm(residual: torch.Tensor, delta: torch.Tensor, w_after: torch.Te
                                   _code(delta, "delta"), nsplit, stride,
                                   _gpu(w_after, "w_after", torch.float32),
                                   _gpu(w_next, "w_next", torch.float32), float(eps),
-                                  _gpu(out, "out"), _code(out, "out"), rows, hidden, _stream())
+                                  _gpu(out, "out"), _code(out, "out"), rows, hidden,
+                                  _row_bias(bias, hidden, "norm_add_norm"), _stream())
     _check(lib, status, "norm_add_norm")
 
 

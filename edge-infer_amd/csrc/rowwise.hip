@@ -420,7 +420,8 @@ namespace {
 template <typename TD, typename TO>
 __global__ void norm_add_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                 int nsplit, size_t split_stride, const float* __restrict__ weight,
-                                float eps, TO* __restrict__ cast_out, int H) {
+                                float eps, TO* __restrict__ cast_out, int H,
+                                const float* __restrict__ bias) {
   extern __shared__ float row_values[];
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * H;
@@ -429,6 +430,7 @@ __global__ void norm_add_kernel(float* __restrict__ residual, const TD* __restri
     const TD* d = delta + base + i;
     float x = 0.f;
     for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TD>(d[s * split_stride]);
+    if (bias) x += bias[i];
     row_values[i] = x;
     sum += x * x;
   }
@@ -447,7 +449,8 @@ template <typename TD, typename TO, int CHUNKS>
 __global__ void norm_add_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                     int nsplit, size_t split_stride,
                                     const float* __restrict__ weight, float eps,
-                                    TO* __restrict__ cast_out, int H) {
+                                    TO* __restrict__ cast_out, int H,
+                                    const float* __restrict__ bias) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * H;
   const int quads = H / 4;
@@ -478,6 +481,12 @@ __global__ void norm_add_vec_kernel(float* __restrict__ residual, const TD* __re
 #pragma unroll
             for (int i = 0; i < 4; ++i) x[k][i] += v[u][i];
           }
+      }
+      if (bias) {
+        float b[4];
+        Vec4<float>::load(bias + qd * 4, b);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[k][i] += b[i];
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) sum += x[k][i] * x[k][i];
@@ -576,7 +585,7 @@ __global__ void activation_vec_kernel(const TI* __restrict__ in, int nsplit, siz
 // new residual rows in out_dtype.
 extern "C" int ei_norm_add(float* residual, const void* delta, int delta_dtype, int nsplit,
                            long long split_stride, const float* weight, float eps, void* cast_out,
-                           int out_dtype, int N, int H, hipStream_t stream) {
+                           int out_dtype, int N, int H, const float* bias, hipStream_t stream) {
   EI_REQUIRE(N > 0 && H > 0, "norm_add: sizes must be positive");
   EI_REQUIRE(H <= 16384, "norm_add: width above 16384 is not supported");
   EI_REQUIRE(residual && delta && weight && nsplit >= 1, "norm_add: bad arguments");
@@ -593,7 +602,8 @@ extern "C" int ei_norm_add(float* residual, const void* delta, int delta_dtype, 
   const int chunks = vec ? (quads + vthreads - 1) / vthreads : 0;      // 1..4 for H <= 16384
 #define EI_NORM_ADD_VEC(TD, TO, C)                                                               \
   norm_add_vec_kernel<TD, TO, C><<<N, vthreads, 0, stream>>>(                                    \
-      residual, static_cast<const TD*>(delta), nsplit, ss, weight, eps, static_cast<TO*>(cast_out), H)
+      residual, static_cast<const TD*>(delta), nsplit, ss, weight, eps, static_cast<TO*>(cast_out), H, \
+      bias)
 #define EI_NORM_ADD(TD, TO)                                                                      \
   do {                                                                                           \
     if (chunks == 1) EI_NORM_ADD_VEC(TD, TO, 1);                                                 \
@@ -602,7 +612,7 @@ extern "C" int ei_norm_add(float* residual, const void* delta, int delta_dtype, 
     else                                                                                         \
       norm_add_kernel<TD, TO><<<N, threads, lds, stream>>>(                                      \
           residual, static_cast<const TD*>(delta), nsplit, ss, weight, eps,                      \
-          static_cast<TO*>(cast_out), H);                                                        \
+          static_cast<TO*>(cast_out), H, bias);                                                  \
   } while (0)
   if (delta_dtype == EI_F32 && (out_dtype == EI_F32 || !cast_out)) EI_NORM_ADD(float, float);
   else if (delta_dtype == EI_F32 && out_dtype == EI_BF16) EI_NORM_ADD(float, bf16_t);
@@ -679,7 +689,8 @@ __global__ void norm_add_norm_kernel(float* __restrict__ residual, const TD* __r
                                      int nsplit, size_t split_stride,
                                      const float* __restrict__ w_after,
                                      const float* __restrict__ w_next, float eps,
-                                     TO* __restrict__ out, int H) {
+                                     TO* __restrict__ out, int H,
+                                     const float* __restrict__ bias) {
   extern __shared__ float row_values[];
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * H;
@@ -688,6 +699,7 @@ __global__ void norm_add_norm_kernel(float* __restrict__ residual, const TD* __r
     const TD* d = delta + base + i;
     float x = 0.f;
     for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TD>(d[s * split_stride]);
+    if (bias) x += bias[i];
     row_values[i] = x;
     sum += x * x;
   }
@@ -711,7 +723,8 @@ __global__ void norm_add_norm_vec_kernel(float* __restrict__ residual, const TD*
                                          int nsplit, size_t split_stride,
                                          const float* __restrict__ w_after,
                                          const float* __restrict__ w_next, float eps,
-                                         TO* __restrict__ out, int H) {
+                                         TO* __restrict__ out, int H,
+                                         const float* __restrict__ bias) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * H;
   const int quads = H / 4;
@@ -743,6 +756,12 @@ __global__ void norm_add_norm_vec_kernel(float* __restrict__ residual, const TD*
 #pragma unroll
             for (int i = 0; i < 4; ++i) x[k][i] += v[u][i];
           }
+      }
+      if (bias) {
+        float b[4];
+        Vec4<float>::load(bias + qd * 4, b);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[k][i] += b[i];
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) sum += x[k][i] * x[k][i];
@@ -810,7 +829,7 @@ __global__ void set_rows_kernel(const TD* __restrict__ x, int nsplit, size_t spl
 extern "C" int ei_norm_add_norm(float* residual, const void* delta, int delta_dtype, int nsplit,
                                 long long split_stride, const float* w_after, const float* w_next,
                                 float eps, void* out, int out_dtype, int N, int H,
-                                hipStream_t stream) {
+                                const float* bias, hipStream_t stream) {
   EI_REQUIRE(N > 0 && H > 0 && nsplit >= 1, "norm_add_norm: sizes must be positive");
   EI_REQUIRE(residual && delta && w_after && w_next && out, "norm_add_norm: null pointer");
   EI_REQUIRE(static_cast<size_t>(H) * sizeof(float) <= 60 * 1024, "norm_add_norm: row too wide");
@@ -827,7 +846,7 @@ extern "C" int ei_norm_add_norm(float* residual, const void* delta, int delta_dt
 #define EI_NAN_VEC(TD, TO, C)                                                                \
   norm_add_norm_vec_kernel<TD, TO, C><<<N, vthreads, 0, stream>>>(                           \
       residual, static_cast<const TD*>(delta), nsplit, ss, w_after, w_next, eps,             \
-      static_cast<TO*>(out), H)
+      static_cast<TO*>(out), H, bias)
 #define EI_NAN_CASE(TD, TO)                                                                  \
   do {                                                                                       \
     if (chunks == 1) EI_NAN_VEC(TD, TO, 1);                                                  \
@@ -836,7 +855,7 @@ extern "C" int ei_norm_add_norm(float* residual, const void* delta, int delta_dt
     else                                                                                     \
       norm_add_norm_kernel<TD, TO><<<N, threads, lds, stream>>>(                             \
           residual, static_cast<const TD*>(delta), nsplit, ss, w_after, w_next, eps,         \
-          static_cast<TO*>(out), H);                                                         \
+          static_cast<TO*>(out), H, bias);                                                   \
   } while (0)
   if (delta_dtype == EI_F32 && out_dtype == EI_F32) EI_NAN_CASE(float, float);
   else if (delta_dtype == EI_F32 && out_dtype == EI_BF16) EI_NAN_CASE(float, bf16_t);

@@ -342,7 +342,11 @@ class Attention:
                 self.decode_launch(n_seqs, pages * PAGE_TOKENS)
         return launch
 
-    def forward(self, ctx, x, entry):
+    bias_later = True      # forward(..., bias_later=True) hands the last product's bias on
+
+    def forward(self, ctx, x, entry, bias_later=False):
+        """The mixer's rows; with `bias_later`, (rows, float32 bias of the output projection
+        that is still to be added, or None), for a caller whose next kernel adds it."""
         spec = self.spec
         n = x.shape[0]
         meta = ctx.meta
@@ -435,6 +439,6 @@ class Attention:
                               spec.n_kv_heads, spec.head_dim, window=spec.window,
                               scale=self.scale, **more)
         ctx.release(qkv, None if isinstance(q, lib.DecodeProjection) else q, part_o, part_ml)
-        delta = self.o.forward(ctx, out, "attn.o")
+        delta = self.o.forward(ctx, out, "attn.o", bias_later=bias_later)
         ctx.release(out)
         return delta

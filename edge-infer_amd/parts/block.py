@@ -276,21 +276,27 @@ class SandwichBlock:
             raise ValueError("sandwich: a delta of the block before is still pending; this "
                              "arrangement follows only blocks that add everything themselves")
         h = self.norm1.add_norm(ctx, residual, None, "block.h", write_residual=False)
-        a = self.mixer.forward(ctx, h, entry)
+        # a sublayer that can leave its last product's bias to the norm kernel behind it does
+        a, a_bias = (self.mixer.forward(ctx, h, entry, bias_later=True)
+                     if getattr(self.mixer, "bias_later", False)
+                     else (self.mixer.forward(ctx, h, entry), None))
         ctx.release(h)
         if self.ffn is None:
-            self.norm1b.norm_add(ctx, residual, a)
+            self.norm1b.norm_add(ctx, residual, a, bias=a_bias)
             ctx.release(a)
             return None
         if self.fused:
             h2 = ctx.buffer("block.h", tuple(residual.shape))
-            lib.norm_add_norm(residual, a, self.norm1b.weight, self.norm2.weight, self.norm2.eps, h2)
+            lib.norm_add_norm(residual, a, self.norm1b.weight, self.norm2.weight, self.norm2.eps, h2,
+                              bias=a_bias)
         else:
-            self.norm1b.norm_add(ctx, residual, a)
+            self.norm1b.norm_add(ctx, residual, a, bias=a_bias)
             h2 = self.norm2.add_norm(ctx, residual, None, "block.h", write_residual=False)
         ctx.release(a)
-        f = self.ffn.forward(ctx, h2)
+        f, f_bias = (self.ffn.forward(ctx, h2, bias_later=True)
+                     if getattr(self.ffn, "bias_later", False)
+                     else (self.ffn.forward(ctx, h2), None))
         ctx.release(h2)
-        self.norm2b.norm_add(ctx, residual, f)
+        self.norm2b.norm_add(ctx, residual, f, bias=f_bias)
         ctx.release(f)
         return None

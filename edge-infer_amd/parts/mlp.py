@@ -78,7 +78,12 @@ class GatedMLP:
         self.down = Linear(params["down_proj.weight"], dtype, device,
                            bias=params.get("down_proj.bias"))
 
-    def forward(self, ctx, x):
+    bias_later = True      # forward(..., bias_later=True) hands the last product's bias on
+
+    def forward(self, ctx, x, bias_later=False):
+        """The feed-forward's rows; with `bias_later`, (rows, float32 bias of the down
+        projection that is still to be added, or None): a caller whose next kernel reads the
+        rows anyway adds it there and saves a launch."""
         n = x.shape[0]
         # (the few-rows product that applies the gate itself knows silu only)
         act = (self.gate_up.forward_gated(ctx, x, "mlp.act")
@@ -89,7 +94,7 @@ class GatedMLP:
             act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
             lib.swiglu(gate_up, act, self.strip, self.spec.activation, bias=bias)
             ctx.release(gate_up)
-        out = self.down.forward(ctx, act, "mlp.down")
+        out = self.down.forward(ctx, act, "mlp.down", bias_later=bias_later)
         ctx.release(act)
         return out
 

@@ -38,12 +38,13 @@ class RMSNorm:
                         write_residual=write_residual)
         return out
 
-    def norm_add(self, ctx, residual, delta, cast_name=None):
-        """residual += rmsnorm(delta) * weight (the norm on a sublayer's output).  With
-        `cast_name`, also returns the new residual rows in the step's storage type, in the
-        buffer of that name (what the next sublayer's product reads)."""
+    def norm_add(self, ctx, residual, delta, cast_name=None, bias=None):
+        """residual += rmsnorm(delta (+ bias)) * weight (the norm on a sublayer's output; `bias`
+        is what the sublayer's last product left to this kernel).  With `cast_name`, also
+        returns the new residual rows in the step's storage type, in the buffer of that name
+        (what the next sublayer's product reads)."""
         cast = None
         if cast_name is not None:
             cast = ctx.buffer(cast_name, tuple(residual.shape))
-        lib.norm_add(residual, delta, self.weight, self.eps, cast_out=cast)
+        lib.norm_add(residual, delta, self.weight, self.eps, cast_out=cast, bias=bias)
         return cast
