@@ -246,7 +246,8 @@ extern "C" int ei_latent_down_store(const void* proj, int in_dtype, int nsplit,
   const int P = q_rank + kv_rank + rot_dim + n_gate;
   const size_t lds = static_cast<size_t>(P) * sizeof(float);
   EI_REQUIRE(lds <= 60 * 1024, "latent_down_store: row too wide");
-  const int threads = 256;
+  // few rows: up to 1024 threads a row, so that a row's loads are in flight together
+  const int threads = N <= 64 ? (P >= 768 ? 1024 : 512) : 256;
   const size_t ss = static_cast<size_t>(split_stride);
 #define EI_LDS_CASE(TI, TO)                                                                     \
   latent_down_store_kernel<TI, TO><<<N, threads, lds, stream>>>(                                \

@@ -102,7 +102,7 @@ _SIGNATURES = {
         "ei_mlstm_proj_width": [c_int, c_int, c_int],
         "ei_mlstm_walk": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p,
                           c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                          c_int, c_int, c_int, c_float, c_float, c_float, c_void_p],
+                          c_int, c_int, c_int, c_float, c_float, c_float, c_int, c_void_p],
         "ei_mlstm_out": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_float,
                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
@@ -740,8 +740,9 @@ def mix_heads(q, talk, out, heads, kv_heads, head_dim) -> None:
 # ---------------------------------------------------------------------------
 # matrix memory (mlstm.hip)
 def mlstm_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
-    """Floats of one sequence's state: per head S^T [value_dim, key_dim], n [key_dim], m."""
-    return heads * (value_dim * key_dim + key_dim + 1)
+    """Floats of one sequence's state: per head S^T [value_dim, key_dim], n [key_dim], m, padded
+    to a multiple of 4 (16-byte accesses)."""
+    return heads * ((value_dim * key_dim + key_dim + 1 + 3) // 4 * 4)
 
 
 def mlstm_proj_width(heads: int, key_dim: int, value_dim: int) -> int:
@@ -774,7 +775,7 @@ def mlstm_walk(proj, i_bias, f_bias, state, seq_in, seq_out, seq_count, seq_row0
         _gpu(seq_in, "seq_in", torch.int32), _gpu(seq_out, "seq_out", torch.int32),
         _gpu(seq_count, "seq_count", torch.int32), _gpu(seq_row0, "seq_row0", torch.int32),
         _gpu(o_raw, "o_raw", torch.float32), n_seqs, heads, key_dim, value_dim, float(cap),
-        float(q_scale), float(bottom_eps), _stream())
+        float(q_scale), float(bottom_eps), n, _stream())
     _check(lib, status, "mlstm_walk")
 
 

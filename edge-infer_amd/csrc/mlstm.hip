@@ -65,6 +65,12 @@ __device__ __forceinline__ float group_sum(float v, int L) {
   return v;
 }
 
+// Floats of one head's state: S^T [vdim, dim], n [dim], m, padded to a multiple of 4 so that
+// every head's part starts at a 16-byte boundary.
+__host__ __device__ inline size_t head_state_floats(int dim, int vdim) {
+  return (static_cast<size_t>(vdim) * dim + dim + 1 + 3) / 4 * 4;
+}
+
 // Column offsets of the fused projection [q | k | v | i | f | g].
 struct Columns {
   int q, k, v, i, f, g, width;
@@ -90,17 +96,19 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
                   const int32_t* __restrict__ seq_in, const int32_t* __restrict__ seq_out,
                   const int32_t* __restrict__ seq_count, const int32_t* __restrict__ seq_row0,
                   float* __restrict__ o_raw, int heads, int dim, int vdim, int L, float cap,
-                  float q_scale, float bottom_eps) {
+                  float q_scale, float bottom_eps, int tile_rows) {
+  // (tile_rows: tokens in LDS at a time, kTile, or 1 where every sequence brings one token: a
+  // decode step then needs a sixteenth of the LDS, and many more waves fit a compute unit)
   extern __shared__ float lds[];
   constexpr int OWN = kOwn;
   const int dimP = L * OWN;
   const int CB = kThreads / L * NC;            // columns of S this block owns
-  float* qs = lds;                             // [kTile][dimP]
-  float* ks = qs + kTile * dimP;               // [kTile][dimP]
-  float* vs = ks + kTile * dimP;               // [kTile][CB]
-  float* keep_s = vs + kTile * CB;             // [kTile] e^(f + m' - m)
-  float* take_s = keep_s + kTile;              // [kTile] e^(i - m)
-  float* floor_s = take_s + kTile;             // [kTile] e^(-m)
+  float* qs = lds;                             // [tile_rows][dimP]
+  float* ks = qs + tile_rows * dimP;           // [tile_rows][dimP]
+  float* vs = ks + tile_rows * dimP;           // [tile_rows][CB]
+  float* keep_s = vs + tile_rows * CB;         // [tile_rows] e^(f + m' - m)
+  float* take_s = keep_s + tile_rows;          // [tile_rows] e^(i - m)
+  float* floor_s = take_s + tile_rows;         // [tile_rows] e^(-m)
 
   const int seq = blockIdx.x / heads, a = blockIdx.x % heads;
   const int count = seq_count[seq];
@@ -112,20 +120,39 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   const int part = t % L, group = t / L;
   const int col0 = blockIdx.y * CB + group * NC;      // the thread's first column
   const int r0 = part * OWN;
-  const size_t head_floats = static_cast<size_t>(vdim) * dim + dim + 1;
+  const size_t head_floats = head_state_floats(dim, vdim);
   const float* in = state + static_cast<size_t>(seq_in[seq]) * state_stride + a * head_floats;
   float* out = state + static_cast<size_t>(seq_out[seq]) * state_stride + a * head_floats;
   // 16-byte loads of q and k: a bfloat16 projection whose head parts start at multiples of 8
   const bool octets = sizeof(TI) == 2 && nsplit == 1 && dim % 8 == 0 && P % 8 == 0;
 
   float S[NC][OWN], nn[OWN];
+  const bool quads = dim % 4 == 0;             // 16-byte accesses to the state
+  if (quads) {
 #pragma unroll
-  for (int r = 0; r < OWN; ++r) {
-    const bool live = r0 + r < dim;
+    for (int r = 0; r < OWN; r += 4) {
+      const bool live = r0 + r < dim;
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
-      S[c][r] = (live && col0 + c < vdim) ? in[static_cast<size_t>(col0 + c) * dim + r0 + r] : 0.f;
-    nn[r] = live ? in[static_cast<size_t>(vdim) * dim + r0 + r] : 0.f;
+      for (int c = 0; c < NC; ++c) {
+        float x[4] = {0.f, 0.f, 0.f, 0.f};
+        if (live && col0 + c < vdim) ei::Vec4<float>::load(in + static_cast<size_t>(col0 + c) * dim + r0 + r, x);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[c][r + e] = x[e];
+      }
+      float x[4] = {0.f, 0.f, 0.f, 0.f};
+      if (live) ei::Vec4<float>::load(in + static_cast<size_t>(vdim) * dim + r0 + r, x);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) nn[r + e] = x[e];
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < OWN; ++r) {
+      const bool live = r0 + r < dim;
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+        S[c][r] = (live && col0 + c < vdim) ? in[static_cast<size_t>(col0 + c) * dim + r0 + r] : 0.f;
+      nn[r] = live ? in[static_cast<size_t>(vdim) * dim + r0 + r] : 0.f;
+    }
   }
   float m_run = in[static_cast<size_t>(vdim) * dim + dim];
 
@@ -135,7 +162,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   const int per_row = dimP / 8;
   const int qk_loads = (kTile * per_row + kThreads - 1) / kThreads;
   const int v_loads = (kTile * CB + kThreads - 1) / kThreads;
-  const bool ahead = octets && qk_loads <= kAhead && v_loads <= kAhead;
+  const bool ahead = octets && tile_rows == kTile && qk_loads <= kAhead && v_loads <= kAhead;
   const bf16_t* rows16 = reinterpret_cast<const bf16_t*>(proj);
   uint4 q_pre[kAhead], k_pre[kAhead];
   bf16_t v_pre[kAhead], xi_pre = 0, xf_pre = 0;
@@ -165,14 +192,14 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
   };
   if (ahead) ask(0);
 
-  for (int t0 = 0; t0 < count; t0 += kTile) {
-    const int tn = min(kTile, count - t0);
+  for (int t0 = 0; t0 < count; t0 += tile_rows) {
+    const int tn = min(tile_rows, count - t0);
     __syncthreads();
     if (ahead) {
 #pragma unroll
       for (int i = 0; i < kAhead; ++i) {
         const int idx = t + i * kThreads;
-        if (i < qk_loads && idx < kTile * per_row) {
+        if (i < qk_loads && idx < tn * per_row) {   // (rows beyond the tile's tokens are never read)
           const int tt = idx / per_row, d = (idx % per_row) * 8;
           const bool live = tt < tn && d < dim;
           const uint32_t qw[4] = {q_pre[i].x, q_pre[i].y, q_pre[i].z, q_pre[i].w};
@@ -189,13 +216,13 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
 #pragma unroll
       for (int i = 0; i < kAhead; ++i) {
         const int idx = t + i * kThreads;
-        if (i < v_loads && idx < kTile * CB) {
+        if (i < v_loads && idx < tn * CB) {
           const bool live = idx / CB < tn && blockIdx.y * CB + idx % CB < vdim;
           vs[idx] = live ? ei::bf16_to_f32(v_pre[i]) : 0.f;
         }
       }
     } else if (octets) {
-      for (int idx = t; idx < kTile * per_row; idx += kThreads) {
+      for (int idx = t; idx < tn * per_row; idx += kThreads) {
         const int tt = idx / per_row, d = (idx % per_row) * 8;
         float qv[8], kv[8];
 #pragma unroll
@@ -212,7 +239,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
         }
       }
     } else {
-      for (int idx = t; idx < kTile * dimP; idx += kThreads) {
+      for (int idx = t; idx < tn * dimP; idx += kThreads) {
         const int tt = idx / dimP, d = idx % dimP;
         float qv = 0.f, kv = 0.f;
         if (tt < tn && d < dim) {
@@ -225,7 +252,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
       }
     }
     if (!ahead) {
-      for (int idx = t; idx < kTile * CB; idx += kThreads) {
+      for (int idx = t; idx < tn * CB; idx += kThreads) {
         const int tt = idx / CB, c = blockIdx.y * CB + idx % CB;
         float v = 0.f;
         if (tt < tn && c < vdim)
@@ -253,7 +280,7 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
         lf = log_sigmoid(cap * tanhf(xf / cap));
       }
       // the next tile's loads travel while this one is walked
-      if (ahead && t0 + kTile < count) ask(t0 + kTile);
+      if (ahead && t0 + kTile < count) ask(t0 + kTile);      // (ahead: tile_rows is kTile)
       float F = lf;                              // sum of the log forget gates up to this token
 #pragma unroll
       for (int step = 1; step < kTile; step *= 2) {
@@ -318,13 +345,29 @@ mlstm_walk_kernel(const TI* __restrict__ proj, int nsplit, size_t split_stride,
     }
   }
 
+  if (quads) {
 #pragma unroll
-  for (int r = 0; r < OWN; ++r) {
-    if (r0 + r < dim) {
+    for (int r = 0; r < OWN; r += 4) {
+      if (r0 + r < dim) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c)
-        if (col0 + c < vdim) out[static_cast<size_t>(col0 + c) * dim + r0 + r] = S[c][r];
-      if (blockIdx.y == 0 && group == 0) out[static_cast<size_t>(vdim) * dim + r0 + r] = nn[r];
+        for (int c = 0; c < NC; ++c) {
+          const float x[4] = {S[c][r], S[c][r + 1], S[c][r + 2], S[c][r + 3]};
+          if (col0 + c < vdim) ei::Vec4<float>::store(out + static_cast<size_t>(col0 + c) * dim + r0 + r, x);
+        }
+        const float x[4] = {nn[r], nn[r + 1], nn[r + 2], nn[r + 3]};
+        if (blockIdx.y == 0 && group == 0)
+          ei::Vec4<float>::store(out + static_cast<size_t>(vdim) * dim + r0 + r, x);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < OWN; ++r) {
+      if (r0 + r < dim) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+          if (col0 + c < vdim) out[static_cast<size_t>(col0 + c) * dim + r0 + r] = S[c][r];
+        if (blockIdx.y == 0 && group == 0) out[static_cast<size_t>(vdim) * dim + r0 + r] = nn[r];
+      }
     }
   }
   if (blockIdx.y == 0 && t == 0) out[static_cast<size_t>(vdim) * dim + dim] = m_run;
@@ -364,9 +407,10 @@ int lanes_for(int dim) {
 
 }  // namespace
 
-// Floats of one sequence's state: per head S^T [vdim, dim], n [dim], m.
+// Floats of one sequence's state: per head S^T [vdim, dim], n [dim], m and padding to a
+// multiple of 4.
 extern "C" int ei_mlstm_state_floats(int heads, int dim, int vdim) {
-  return heads * (vdim * dim + dim + 1);
+  return heads * static_cast<int>(head_state_floats(dim, vdim));
 }
 
 // Width of the fused projection [q | k | v | i | f | g].
@@ -381,15 +425,15 @@ extern "C" int ei_mlstm_walk(const void* proj, int dtype, int nsplit, long long 
                              long long state_stride, const int32_t* seq_in, const int32_t* seq_out,
                              const int32_t* seq_count, const int32_t* seq_row0, float* o_raw,
                              int n_seqs, int heads, int dim, int vdim, float cap, float q_scale,
-                             float bottom_eps, hipStream_t stream) {
-  EI_REQUIRE(n_seqs > 0 && heads > 0 && vdim > 0 && nsplit >= 1, "mlstm_walk: bad sizes");
+                             float bottom_eps, int rows, hipStream_t stream) {
+  EI_REQUIRE(n_seqs > 0 && heads > 0 && vdim > 0 && nsplit >= 1 && rows >= 1, "mlstm_walk: bad sizes");
   EI_REQUIRE(dim >= 1 && dim <= 256, "mlstm_walk: the key size must lie in 1..256");
   EI_REQUIRE(cap > 0.f, "mlstm_walk: the cap of the gates must be positive");
   EI_REQUIRE(proj && i_bias && f_bias && state && seq_in && seq_out && seq_count && seq_row0 &&
                  o_raw,
              "mlstm_walk: null pointer");
-  EI_REQUIRE(state_stride >= ei_mlstm_state_floats(heads, dim, vdim),
-             "mlstm_walk: state rows too short");
+  EI_REQUIRE(state_stride >= ei_mlstm_state_floats(heads, dim, vdim) && state_stride % 4 == 0,
+             "mlstm_walk: state rows too short, or no multiple of 4 floats");
   const int L = lanes_for(dim);
   // columns a thread: as many (4, 2, 1) as still give every SIMD of the chip two waves
   const long long wanted = 2LL * 4 * ei_compute_units();
@@ -398,8 +442,10 @@ extern "C" int ei_mlstm_walk(const void* proj, int dtype, int nsplit, long long 
                            ((vdim + kThreads / L * nc - 1) / (kThreads / L * nc)) < wanted)
     nc /= 2;
   const int CB = kThreads / L * nc;
-  const size_t lds = sizeof(float) * (2 * static_cast<size_t>(kTile) * L * kOwn +
-                                      static_cast<size_t>(kTile) * CB + 3 * kTile);
+  // no more rows than sequences: every sequence brings one token at most (a decode step)
+  const int tile_rows = rows <= n_seqs ? 1 : kTile;
+  const size_t lds = sizeof(float) * (2 * static_cast<size_t>(tile_rows) * L * kOwn +
+                                      static_cast<size_t>(tile_rows) * CB + 3 * tile_rows);
   EI_REQUIRE(static_cast<long long>(n_seqs) * heads <= 0x7fffffffLL, "mlstm_walk: too many blocks");
   EI_REQUIRE((vdim + CB - 1) / CB <= 65535, "mlstm_walk: too many blocks of columns");
   dim3 grid(n_seqs * heads, (vdim + CB - 1) / CB);
@@ -408,7 +454,7 @@ extern "C" int ei_mlstm_walk(const void* proj, int dtype, int nsplit, long long 
   mlstm_walk_kernel<TI, NC><<<grid, kThreads, lds, stream>>>(                                  \
       static_cast<const TI*>(proj), nsplit, ss, i_bias, f_bias, state,                         \
       static_cast<size_t>(state_stride), seq_in, seq_out, seq_count, seq_row0, o_raw, heads,   \
-      dim, vdim, L, cap, q_scale, bottom_eps)
+      dim, vdim, L, cap, q_scale, bottom_eps, tile_rows)
 #define EI_WALK_COLS(TI)              \
   do {                                \
     if (nc == 4) EI_WALK(TI, 4);      \

@@ -143,9 +143,9 @@ class LatentAttention:
         """Slices of the key range in a decode step: enough blocks for about two a compute
         unit, never more than there are pages."""
         pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
-        if self.wide:         # blocks of up to 64 heads, about one a compute unit
+        if self.wide:         # blocks of up to 64 heads, about two a compute unit
             blocks = n_seqs * ((self.spec.n_heads + 63) // 64)
-            wanted = max(1, self.compute_units // blocks)
+            wanted = max(1, 2 * self.compute_units // blocks)
         else:
             blocks = n_seqs * ((self.spec.n_heads + 15) // 16)
             wanted = (2 * self.compute_units + blocks - 1) // blocks

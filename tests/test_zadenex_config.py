@@ -156,7 +156,7 @@ def test_cache_requests():
     by_request = {request: entries for request, entries in layout.kv_groups}
     assert by_request[KVRequest(n_kv_heads=1, head_dim=48, value_dim=0)] == [1, 3, 5]   # three passes
     (state, entries), = layout.state_groups
-    assert state == StateRequest(shape=(3 * (16 * 24 + 24 + 1),), two_versions=True)
+    assert state == StateRequest(shape=(3 * 412,), two_versions=True)      # 16 * 24 + 24 + 1, padded to 4
     assert entries == [2, 4, 6]
 
 
