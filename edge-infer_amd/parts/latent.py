@@ -1,6 +1,6 @@
 """Causal attention over a latent cache: per position one normed latent vector c [kv_rank],
 from which every head's unrotated key and its value are up-projections, and one rotated key
-part [rot_dim] that all heads share.  Only c and the rotated part are cached.
+part [rot_dim] that all heads share.  The cache holds nothing but c and that part.
 
 With x the mixer's input, head a, W_uk,a [head_dim, kv_rank] and W_uv,a [value_dim, kv_rank]
 the head's rows of the two up-projections:
