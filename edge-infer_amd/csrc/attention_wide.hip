@@ -30,6 +30,7 @@ constexpr int kRows = 64;         // query rows of a block
 constexpr int kKeys = 32;         // keys of a tile
 constexpr int kPadK = 8;          // elements of padding of a key row in LDS
 constexpr int kVtRow = kKeys + 8; // elements of a row of the transposed values in LDS
+constexpr int kBatch = 5;         // loads of a tile that a thread has in flight together
 constexpr float kLowest = -1.0e30f;
 
 template <int NK, int NDV>
@@ -101,38 +102,65 @@ attn_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_page
       if (key0 > hi_key) break;
       if (key0 + kKeys <= lo_key) continue;
       __syncthreads();
-      // keys as stored; with values inside the keys, their first DV elements transposed as well
-      // (neighbouring lanes take neighbouring keys: their 2-byte writes of the transposed
-      // values then fall into 32 banks, two lanes a word, instead of into two banks)
-      for (int ch = t; ch < kKeys * k_chunks; ch += kThreads) {
-        const int key = ch % kKeys, col = (ch / kKeys) * 8;
-        const int kh = KH > 1 ? col / D : g, dd = KH > 1 ? col % D : col;
-        uint4 val = uint4{0u, 0u, 0u, 0u};
-        if (key0 + key <= hi_key)       // later slots hold stale bytes
-          val = *reinterpret_cast<const uint4*>(
-              k_pages + ((static_cast<size_t>(phys) * nkv + kh) * EI_PAGE + half * kKeys + key) * D + dd);
-        *reinterpret_cast<uint4*>(Kt + key * k_row + col) = val;
-        if (values_in_keys && col < DV) {
-          const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+      // keys as stored; with values inside the keys, their first DV elements transposed as well.
+      // Neighbouring lanes take neighbouring keys: their 2-byte writes of the transposed values
+      // then fall into 32 banks, two lanes a word, instead of into two banks.  The loads of a
+      // batch are unconditional, from clamped places (a live key of the tile, the last chunk),
+      // so that they travel together instead of each waiting behind a branch.
+      const int last_live = min(kKeys - 1, hi_key - key0);
+      const int k_total = kKeys * k_chunks;
+      for (int base = 0; base < k_total; base += kThreads * kBatch) {
+        uint4 val[kBatch];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            Vt[(col + 2 * i) * kVtRow + key] = static_cast<bf16_t>(w[i] & 0xffffu);
-            Vt[(col + 2 * i + 1) * kVtRow + key] = static_cast<bf16_t>(w[i] >> 16);
+        for (int u = 0; u < kBatch; ++u) {
+          const int ch = min(base + u * kThreads + t, k_total - 1);
+          const int key = min(ch % kKeys, last_live), col = (ch / kKeys) * 8;
+          const int kh = KH > 1 ? col / D : g, dd = KH > 1 ? col % D : col;
+          val[u] = *reinterpret_cast<const uint4*>(
+              k_pages + ((static_cast<size_t>(phys) * nkv + kh) * EI_PAGE + half * kKeys + key) * D + dd);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int ch = base + u * kThreads + t;
+          if (ch < k_total) {
+            const int key = ch % kKeys, col = (ch / kKeys) * 8;
+            const uint4 v = key <= last_live ? val[u] : uint4{0u, 0u, 0u, 0u};   // stale slots: zeros
+            *reinterpret_cast<uint4*>(Kt + key * k_row + col) = v;
+            if (values_in_keys && col < DV) {
+              const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                Vt[(col + 2 * i) * kVtRow + key] = static_cast<bf16_t>(w[i] & 0xffffu);
+                Vt[(col + 2 * i + 1) * kVtRow + key] = static_cast<bf16_t>(w[i] >> 16);
+              }
+            }
           }
         }
       }
       if (!values_in_keys) {
-        for (int ch = t; ch < kKeys * v_chunks; ch += kThreads) {
-          const int key = ch % kKeys, col = (ch / kKeys) * 8;
-          uint4 val = uint4{0u, 0u, 0u, 0u};
-          if (key0 + key <= hi_key)
-            val = *reinterpret_cast<const uint4*>(
-                v_pages + ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + half * kKeys + key) * DV + col);
-          const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+        const int v_total = kKeys * v_chunks;
+        for (int base = 0; base < v_total; base += kThreads * kBatch) {
+          uint4 val[kBatch];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            Vt[(col + 2 * i) * kVtRow + key] = static_cast<bf16_t>(w[i] & 0xffffu);
-            Vt[(col + 2 * i + 1) * kVtRow + key] = static_cast<bf16_t>(w[i] >> 16);
+          for (int u = 0; u < kBatch; ++u) {
+            const int ch = min(base + u * kThreads + t, v_total - 1);
+            const int key = min(ch % kKeys, last_live), col = (ch / kKeys) * 8;
+            val[u] = *reinterpret_cast<const uint4*>(
+                v_pages + ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + half * kKeys + key) * DV + col);
+          }
+#pragma unroll
+          for (int u = 0; u < kBatch; ++u) {
+            const int ch = base + u * kThreads + t;
+            if (ch < v_total) {
+              const int key = ch % kKeys, col = (ch / kKeys) * 8;
+              const uint4 v = key <= last_live ? val[u] : uint4{0u, 0u, 0u, 0u};
+              const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                Vt[(col + 2 * i) * kVtRow + key] = static_cast<bf16_t>(w[i] & 0xffffu);
+                Vt[(col + 2 * i + 1) * kVtRow + key] = static_cast<bf16_t>(w[i] >> 16);
+              }
+            }
           }
         }
       }
