@@ -30,7 +30,6 @@ constexpr int kRows = 64;         // query rows of a block
 constexpr int kKeys = 32;         // keys of a tile
 constexpr int kPadK = 8;          // elements of padding of a key row in LDS
 constexpr int kVtRow = kKeys + 8; // elements of a row of the transposed values in LDS
-constexpr int kBatch = 5;         // loads of a tile that a thread has in flight together
 constexpr float kLowest = -1.0e30f;
 
 template <int NK, int NDV>
@@ -107,6 +106,8 @@ attn_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_page
       // then fall into 32 banks, two lanes a word, instead of into two banks.  The loads of a
       // batch are unconditional, from clamped places (a live key of the tile, the last chunk),
       // so that they travel together instead of each waiting behind a branch.
+      // (the widest query rows leave no registers for it: two waves a SIMD count for more there)
+      constexpr int kBatch = NK > 18 ? 1 : 5;
       const int last_live = min(kKeys - 1, hi_key - key0);
       const int k_total = kKeys * k_chunks;
       for (int base = 0; base < k_total; base += kThreads * kBatch) {
